@@ -1,0 +1,20 @@
+"""MI355X-native fused Mixture-of-Experts layer behind fast-route's entry points.
+
+Host code is PyTorch-ROCm (device memory and streams only); all compute is in
+hand-written HIP kernels for gfx950, reached through the C ABI declared in
+include/fast_route_hip.h.  There is no CPU or eager fallback: every operator
+raises if the native library is missing.
+"""
+from . import _native  # noqa: F401
+from .layers.fused_moe import fused_moe, fused_experts  # noqa: F401
+from .ops.fused_moe import moe_align_block_size, invoke_fused_moe_kernel  # noqa: F401
+from .ops.stable_route import fused_route, topk_softmax  # noqa: F401
+
+__all__ = [
+    "fused_moe",
+    "fused_experts",
+    "moe_align_block_size",
+    "invoke_fused_moe_kernel",
+    "fused_route",
+    "topk_softmax",
+]

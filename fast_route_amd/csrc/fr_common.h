@@ -1,0 +1,61 @@
+// Shared host/device helpers for the gfx950 fused-MoE kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "fast_route_hip.h"
+
+namespace fr {
+
+// ---- error reporting (thread local, never throws) -------------------------
+char* error_buffer();
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+#define FR_REQUIRE(cond, code, ...) \
+  do {                              \
+    if (!(cond)) return ::fr::fail((code), __VA_ARGS__); \
+  } while (0)
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
+
+// ---- device-side scalar types ---------------------------------------------
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+template <typename T>
+__device__ __forceinline__ float to_float(T v) { return static_cast<float>(v); }
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kWave = 64;
+
+// ---- cross-lane exchange ----------------------------------------------------
+// partner<S>(v): value held by this lane's partner at butterfly step S.  Steps
+// 1 and 2 are DPP quad permutes, 4 and 8 DPP mirrors inside a row of 16 lanes
+// (an involution that pairs the two halves, which is all an all-reduce needs),
+// 16 and 32 go through the LDS crossbar.
+template <int S>
+__device__ __forceinline__ int partner_i32(int v) {
+  if constexpr (S == 1) return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+  else if constexpr (S == 2) return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+  else if constexpr (S == 4) return __builtin_amdgcn_update_dpp(v, v, 0x141, 0xF, 0xF, false); // row_half_mirror
+  else if constexpr (S == 8) return __builtin_amdgcn_update_dpp(v, v, 0x140, 0xF, 0xF, false); // row_mirror
+  else return __shfl_xor(v, S, kWave);
+}
+template <int S>
+__device__ __forceinline__ float partner_f32(float v) {
+  return __int_as_float(partner_i32<S>(__float_as_int(v)));
+}
+
+}  // namespace fr

@@ -1,0 +1,116 @@
+// Composite entry points: tile plan, workspace carving, and the whole layer as
+// one sequence of launches on the caller's stream.
+#include "fr_common.h"
+
+namespace fr {
+namespace {
+
+constexpr int64_t kAlign = 256;
+int64_t aligned(int64_t bytes) { return round_up(bytes, kAlign); }
+
+struct Carve {
+  float* topk_w;
+  int32_t* topk_ids;
+  int32_t* sorted;
+  int32_t* expert_ids;
+  int32_t* npost;
+  void* align_ws;
+  int64_t align_ws_bytes;
+  void* act;
+  float* partial;
+  int64_t total;
+};
+
+int elem_size(int dtype) { return (dtype == FR_F16 || dtype == FR_BF16) ? 2 : (dtype == FR_F32 ? 4 : 1); }
+
+Carve carve(void* base, int64_t M, int64_t H, int64_t F, int E, int topk, int dtype, const fr_moe_plan& p) {
+  Carve c;
+  const int64_t n = M * topk;
+  char* b = static_cast<char*>(base);
+  int64_t off = 0;
+  auto take = [&](int64_t bytes) { char* r = b ? b + off : nullptr; off += aligned(bytes); return r; };
+  c.topk_w = reinterpret_cast<float*>(take(n * 4));
+  c.topk_ids = reinterpret_cast<int32_t*>(take(n * 4));
+  c.sorted = reinterpret_cast<int32_t*>(take(p.sorted_len * 4));
+  c.expert_ids = reinterpret_cast<int32_t*>(take((n + E) * 4));
+  c.npost = reinterpret_cast<int32_t*>(take(4));
+  c.align_ws_bytes = fr_moe_align_workspace_bytes(n, E);
+  c.align_ws = take(c.align_ws_bytes);
+  c.act = take(p.sorted_len * F * elem_size(dtype));
+  c.partial = reinterpret_cast<float*>(take(static_cast<int64_t>(p.split_k) * n * H * 4));
+  c.total = off;
+  return c;
+}
+
+int check_layer_shapes(const char* who, int64_t M, int64_t H, int64_t F, int E, int topk, int dtype) {
+  FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "%s: dtype %d not in {f16, bf16}", who, dtype);
+  FR_REQUIRE(M >= 0 && H > 0 && F > 0, FR_E_SHAPE, "%s: M=%lld H=%lld F=%lld", who, (long long)M, (long long)H, (long long)F);
+  FR_REQUIRE(E >= 1 && E <= 1024 && topk >= 1 && topk <= E, FR_E_SHAPE, "%s: E=%d topk=%d", who, E, topk);
+  FR_REQUIRE(H % 128 == 0 && F % 128 == 0, FR_E_SHAPE, "%s: H=%lld and F=%lld must be multiples of 128", who, (long long)H, (long long)F);
+  FR_REQUIRE(M * topk < (int64_t(1) << 30), FR_E_SHAPE, "%s: M*topk too large", who);
+  return FR_OK;
+}
+
+}  // namespace
+}  // namespace fr
+
+using namespace fr;
+
+extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk, int dtype, fr_moe_plan* plan) {
+  FR_REQUIRE(plan, FR_E_NULL, "fr_moe_get_plan: null plan");
+  int rc = check_layer_shapes("fr_moe_get_plan", M, H, F, E, topk, dtype);
+  if (rc != FR_OK) return rc;
+  const int64_t n = M * topk;
+  const double avg = static_cast<double>(n) / E;  // expected pairs per expert under uniform load
+  int block;
+  if (avg <= 8) block = 16;
+  else if (avg <= 24) block = 32;
+  else if (avg <= 64) block = 64;
+  else block = 128;
+  // down projection: few feature tiles (N = H), so split K until the grid covers the chip
+  const int bf = block >= 64 ? 256 : 128;
+  const int64_t active_blocks = n < E ? n : (block >= 64 ? ceil_div(n, block) + E / 2 : E);
+  const int64_t tiles = active_blocks * ceil_div(H, bf);
+  int split = 1;
+  const int bk = block >= 64 ? 64 : 128;
+  while (split < 16 && tiles * split < 1024 && F / (split * 2) >= 4 * bk) split *= 2;
+  plan->block = block;
+  plan->split_k = split;
+  plan->sorted_len = n + static_cast<int64_t>(E) * (block - 1);
+  plan->workspace_bytes = carve(nullptr, M, H, F, E, topk, dtype, *plan).total;
+  return FR_OK;
+}
+
+extern "C" int fr_fused_experts(const void* x, const void* w1, const void* w2, const float* topk_weights,
+                                const int32_t* topk_ids, int64_t M, int64_t H, int64_t F, int E, int topk,
+                                int dtype, void* out, void* workspace, int64_t workspace_bytes, void* stream) {
+  fr_moe_plan p;
+  int rc = fr_moe_get_plan(M, H, F, E, topk, dtype, &p);
+  if (rc != FR_OK) return rc;
+  if (M == 0) return FR_OK;
+  FR_REQUIRE(x && w1 && w2 && topk_weights && topk_ids && out, FR_E_NULL, "fr_fused_experts: null pointer");
+  FR_REQUIRE(workspace && workspace_bytes >= p.workspace_bytes, FR_E_WORKSPACE, "fr_fused_experts: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)p.workspace_bytes);
+  FR_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FR_E_ALIGN, "fr_fused_experts: workspace must be 256-byte aligned");
+  Carve c = carve(workspace, M, H, F, E, topk, dtype, p);
+  rc = fr_moe_align(topk_ids, FR_I32, M * topk, E, p.block, c.sorted, c.expert_ids, c.npost, c.align_ws, c.align_ws_bytes, stream);
+  if (rc != FR_OK) return rc;
+  rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, stream);
+  if (rc != FR_OK) return rc;
+  return fr_moe_down_combine(c.act, w2, topk_weights, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, p.split_k, dtype, c.partial, out, stream);
+}
+
+extern "C" int fr_fused_moe(const void* x, const void* w1, const void* w2, const void* logits, int logits_dtype,
+                            int64_t M, int64_t H, int64_t F, int E, int topk, int renormalize, int dtype,
+                            void* out, void* workspace, int64_t workspace_bytes, void* stream) {
+  fr_moe_plan p;
+  int rc = fr_moe_get_plan(M, H, F, E, topk, dtype, &p);
+  if (rc != FR_OK) return rc;
+  if (M == 0) return FR_OK;
+  FR_REQUIRE(x && w1 && w2 && logits && out, FR_E_NULL, "fr_fused_moe: null pointer");
+  FR_REQUIRE(workspace && workspace_bytes >= p.workspace_bytes, FR_E_WORKSPACE, "fr_fused_moe: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)p.workspace_bytes);
+  FR_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FR_E_ALIGN, "fr_fused_moe: workspace must be 256-byte aligned");
+  Carve c = carve(workspace, M, H, F, E, topk, dtype, p);
+  rc = fr_gating_topk(logits, logits_dtype, M, E, E, topk, renormalize, c.topk_w, c.topk_ids, stream);
+  if (rc != FR_OK) return rc;
+  return fr_fused_experts(x, w1, w2, c.topk_w, c.topk_ids, M, H, F, E, topk, dtype, out, workspace, workspace_bytes, stream);
+}

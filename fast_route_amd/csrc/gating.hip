@@ -1,0 +1,311 @@
+// Top-k gating for router logits on gfx950.
+//
+// A group of G lanes (G = next power of two >= E, at most one wavefront) owns
+// one token; each lane keeps VPL logits in registers (expert = lane + i*G), so
+// a wavefront handles 64/G tokens.  Softmax statistics use the online
+// (max, sum) recurrence combined across lanes with one butterfly; top-k is k
+// rounds of a cross-lane arg-max under the total order (value descending,
+// expert index ascending), which is what a stable descending sort yields.
+#include "fr_common.h"
+
+#include <float.h>
+#include <limits.h>
+
+#include <type_traits>
+
+namespace fr {
+namespace {
+
+__device__ __forceinline__ bool better(float av, int ai, float bv, int bi) {
+  return av > bv || (av == bv && ai < bi);
+}
+
+template <int G>
+__device__ __forceinline__ void group_online_softmax(float& m, float& s) {
+  auto step = [&](auto tag) {
+    constexpr int S = decltype(tag)::value;
+    const float m2 = partner_f32<S>(m);
+    const float s2 = partner_f32<S>(s);
+    const float mn = fmaxf(m, m2);
+    const float a = (m == -INFINITY) ? 0.f : s * expf(m - mn);
+    const float b = (m2 == -INFINITY) ? 0.f : s2 * expf(m2 - mn);
+    // a + b is evaluated with the lower lane's term first in both partners so
+    // every lane of the group ends with bit-identical statistics
+    const bool low = (static_cast<int>(threadIdx.x) & S) == 0;
+    s = low ? (a + b) : (b + a);
+    m = mn;
+  };
+  if constexpr (G > 1) step(std::integral_constant<int, 1>{});
+  if constexpr (G > 2) step(std::integral_constant<int, 2>{});
+  if constexpr (G > 4) step(std::integral_constant<int, 4>{});
+  if constexpr (G > 8) step(std::integral_constant<int, 8>{});
+  if constexpr (G > 16) step(std::integral_constant<int, 16>{});
+  if constexpr (G > 32) step(std::integral_constant<int, 32>{});
+}
+
+template <int G>
+__device__ __forceinline__ void group_argmax(float& v, int& i) {
+  auto step = [&](auto tag) {
+    constexpr int S = decltype(tag)::value;
+    const float ov = partner_f32<S>(v);
+    const int oi = partner_i32<S>(i);
+    if (better(ov, oi, v, i)) {
+      v = ov;
+      i = oi;
+    }
+  };
+  if constexpr (G > 1) step(std::integral_constant<int, 1>{});
+  if constexpr (G > 2) step(std::integral_constant<int, 2>{});
+  if constexpr (G > 4) step(std::integral_constant<int, 4>{});
+  if constexpr (G > 8) step(std::integral_constant<int, 8>{});
+  if constexpr (G > 16) step(std::integral_constant<int, 16>{});
+  if constexpr (G > 32) step(std::integral_constant<int, 32>{});
+}
+
+constexpr int kGateThreads = 256;
+
+// Gating of one token by a group of G lanes.  `load(e)` returns logit e as fp32;
+// every lane of the wavefront must call this (dead groups pass live = false).
+template <int G, int VPL, typename Load>
+__device__ __forceinline__ void gate_token(Load load, bool live, int E, int topk, int renorm,
+                                           float* __restrict__ w_row, int32_t* __restrict__ id_row) {
+  const int g = threadIdx.x % G;
+  float v[VPL];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int e = g + i * G;
+    v[i] = (live && e < E) ? load(e) : -INFINITY;
+  }
+
+  // online softmax statistics over this lane's values, then across the group
+  float m = v[0];
+#pragma unroll
+  for (int i = 1; i < VPL; ++i) m = fmaxf(m, v[i]);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) s += (v[i] == -INFINITY) ? 0.f : expf(v[i] - m);
+  group_online_softmax<G>(m, s);
+
+  float sel_v[VPL];
+  int sel_i[VPL];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    sel_v[i] = -INFINITY;
+    sel_i[i] = 0;
+  }
+  unsigned taken = 0;
+  float sel_sum = 0.f;
+  for (int r = 0; r < topk; ++r) {
+    float bv = -INFINITY;
+    int bi = INT_MAX;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int e = g + i * G;
+      if (e < E && !((taken >> i) & 1u) && better(v[i], e, bv, bi)) {
+        bv = v[i];
+        bi = e;
+      }
+    }
+    group_argmax<G>(bv, bi);
+    if (bi % G == g) taken |= 1u << (bi / G);
+    sel_sum += expf(bv - m);
+#pragma unroll
+    for (int sl = 0; sl < VPL; ++sl) {
+      if (r == sl * G + g) {
+        sel_v[sl] = bv;
+        sel_i[sl] = bi;
+      }
+    }
+  }
+
+  const float denom = renorm ? sel_sum : s;
+  if (live) {
+#pragma unroll
+    for (int sl = 0; sl < VPL; ++sl) {
+      const int r = sl * G + g;
+      if (r < topk) {
+        w_row[r] = expf(sel_v[sl] - m) / denom;
+        id_row[r] = sel_i[sl];
+      }
+    }
+  }
+}
+
+template <typename T, int G, int VPL>
+__global__ __launch_bounds__(kGateThreads) void gating_topk_kernel(
+    const T* __restrict__ logits, int64_t M, int E, int64_t ld, int topk, int renorm,
+    float* __restrict__ w_out, int32_t* __restrict__ ids_out) {
+  const int64_t token = (static_cast<int64_t>(blockIdx.x) * kGateThreads + threadIdx.x) / G;
+  const bool live = token < M;
+  const T* row = logits + (live ? token : 0) * ld;
+  gate_token<G, VPL>([&](int e) { return to_float(row[e]); }, live, E, topk, renorm,
+                     w_out + token * topk, ids_out + token * topk);
+}
+
+// ---- gate-matrix form: logits tile by MFMA, then the same gating -------------
+// One workgroup owns kRgTokens tokens (16 per wavefront).  The gate matrix is
+// [H, E] with experts contiguous, so each K tile of it is transposed through
+// LDS into expert-major rows that the MFMA "A" operand can read as 16-byte
+// vectors; token rows come straight from HBM as the "B" operand.
+constexpr int kRgTokens = 64;
+constexpr int kRgBK = 64;
+constexpr int kRgPitch = kRgBK + 8;  // elements; keeps 16-byte alignment, spreads banks
+constexpr int kRgMaxE = 64;
+
+template <typename T> struct Mfma16;
+template <> struct Mfma16<bf16_t> {
+  typedef bf16x8 vec8;
+  static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct Mfma16<f16_t> {
+  typedef f16x8 vec8;
+  static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+};
+
+template <typename T, int G>
+__global__ __launch_bounds__(kGateThreads) void route_gate_kernel(
+    const T* __restrict__ hidden, const T* __restrict__ gate, int64_t M, int H, int E, int topk,
+    int renorm, float* __restrict__ w_out, int32_t* __restrict__ ids_out) {
+  typedef typename Mfma16<T>::vec8 vec8;
+  constexpr int ET = (G + 15) / 16;  // expert tiles of 16
+  __shared__ __attribute__((aligned(16))) T gt[ET * 16 * kRgPitch];
+  __shared__ float logit[kRgTokens * (kRgMaxE + 1)];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * kRgTokens;
+  const int64_t my_tok = tok0 + wave * 16 + (lane & 15);
+  const T* xrow = hidden + (my_tok < M ? my_tok : 0) * H + (lane >> 4) * 8;
+
+  for (int i = tid; i < ET * 16 * kRgPitch; i += kGateThreads) gt[i] = static_cast<T>(0.f);
+  f32x4 acc[ET];
+#pragma unroll
+  for (int j = 0; j < ET; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int k0 = 0; k0 < H; k0 += kRgBK) {
+    __syncthreads();
+    const int kmax = min(kRgBK, H - k0);
+    for (int i = tid; i < kmax * E; i += kGateThreads) {
+      const int k = i / E, e = i % E;
+      gt[e * kRgPitch + k] = gate[static_cast<int64_t>(k0 + k) * E + e];
+    }
+    if (kmax < kRgBK)
+      for (int i = tid; i < (kRgBK - kmax) * E; i += kGateThreads) gt[(i % E) * kRgPitch + kmax + i / E] = static_cast<T>(0.f);
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < kRgBK / 32; ++ks) {
+      const int kk = k0 + ks * 32 + (lane >> 4) * 8;
+      vec8 xf;
+      if (kk + 8 <= H) xf = *reinterpret_cast<const vec8*>(xrow + k0 + ks * 32);
+      else
+#pragma unroll
+        for (int r = 0; r < 8; ++r) xf[r] = static_cast<T>(0.f);
+#pragma unroll
+      for (int j = 0; j < ET; ++j) {
+        const vec8 gf = *reinterpret_cast<const vec8*>(&gt[(j * 16 + (lane & 15)) * kRgPitch + ks * 32 + (lane >> 4) * 8]);
+        acc[j] = Mfma16<T>::mma(gf, xf, acc[j]);
+      }
+    }
+  }
+  // accumulator rows are experts (lane/16*4 + r inside tile j), columns tokens
+#pragma unroll
+  for (int j = 0; j < ET; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int e = j * 16 + (lane >> 4) * 4 + r;
+      if (e < E) logit[(wave * 16 + (lane & 15)) * (kRgMaxE + 1) + e] = acc[j][r];
+    }
+  __syncthreads();
+  constexpr int PER_PASS = kGateThreads / G;
+  for (int t = tid / G; t < kRgTokens; t += PER_PASS) {
+    const int64_t token = tok0 + t;
+    const bool live = token < M;
+    const float* row = logit + t * (kRgMaxE + 1);
+    gate_token<G, 1>([&](int e) { return row[e]; }, live, E, topk, renorm, w_out + token * topk,
+                     ids_out + token * topk);
+  }
+}
+
+template <typename T, int G, int VPL>
+void launch(const void* logits, int64_t M, int E, int64_t ld, int topk, int renorm, float* w,
+            int32_t* ids, hipStream_t st) {
+  const int64_t tokens_per_block = kGateThreads / G;
+  const unsigned grid = static_cast<unsigned>(ceil_div(M, tokens_per_block));
+  hipLaunchKernelGGL((gating_topk_kernel<T, G, VPL>), dim3(grid), dim3(kGateThreads), 0, st,
+                     static_cast<const T*>(logits), M, E, ld, topk, renorm, w, ids);
+}
+
+template <typename T>
+int dispatch(const void* logits, int64_t M, int E, int64_t ld, int topk, int renorm, float* w,
+             int32_t* ids, hipStream_t st) {
+  if (E <= 1) launch<T, 1, 1>(logits, M, E, ld, topk, renorm, w, ids, st);
+  else if (E <= 2) launch<T, 2, 1>(logits, M, E, ld, topk, renorm, w, ids, st);
+  else if (E <= 4) launch<T, 4, 1>(logits, M, E, ld, topk, renorm, w, ids, st);
+  else if (E <= 8) launch<T, 8, 1>(logits, M, E, ld, topk, renorm, w, ids, st);
+  else if (E <= 16) launch<T, 16, 1>(logits, M, E, ld, topk, renorm, w, ids, st);
+  else if (E <= 32) launch<T, 32, 1>(logits, M, E, ld, topk, renorm, w, ids, st);
+  else if (E <= 64) launch<T, 64, 1>(logits, M, E, ld, topk, renorm, w, ids, st);
+  else if (E <= 128) launch<T, 64, 2>(logits, M, E, ld, topk, renorm, w, ids, st);
+  else launch<T, 64, 4>(logits, M, E, ld, topk, renorm, w, ids, st);
+  return check_launch("gating_topk_kernel");
+}
+
+}  // namespace
+}  // namespace fr
+
+extern "C" int fr_gating_topk(const void* logits, int logits_dtype, int64_t M, int64_t E,
+                              int64_t ld, int topk, int renormalize, float* weights_out,
+                              int32_t* ids_out, void* stream) {
+  using namespace fr;
+  FR_REQUIRE(M >= 0, FR_E_SHAPE, "fr_gating_topk: M=%lld < 0", (long long)M);
+  if (M == 0) return FR_OK;
+  FR_REQUIRE(logits && weights_out && ids_out, FR_E_NULL, "fr_gating_topk: null pointer");
+  FR_REQUIRE(E >= 1 && E <= 256, FR_E_SHAPE, "fr_gating_topk: E=%lld outside [1, 256]", (long long)E);
+  FR_REQUIRE(topk >= 1 && topk <= E, FR_E_SHAPE, "fr_gating_topk: topk=%d outside [1, E=%lld]", topk, (long long)E);
+  FR_REQUIRE(ld >= E, FR_E_SHAPE, "fr_gating_topk: row stride %lld < E", (long long)ld);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (logits_dtype) {
+    case FR_F32: return dispatch<float>(logits, M, (int)E, ld, topk, renormalize, weights_out, ids_out, st);
+    case FR_F16: return dispatch<f16_t>(logits, M, (int)E, ld, topk, renormalize, weights_out, ids_out, st);
+    case FR_BF16: return dispatch<bf16_t>(logits, M, (int)E, ld, topk, renormalize, weights_out, ids_out, st);
+    default: return fail(FR_E_DTYPE, "fr_gating_topk: logits dtype %d not in {f16, bf16, f32}", logits_dtype);
+  }
+}
+
+namespace fr {
+namespace {
+template <typename T, int G>
+void launch_route_gate(const void* hidden, const void* gate, int64_t M, int H, int E, int topk, int renorm,
+                       float* w, int32_t* ids, hipStream_t st) {
+  const unsigned grid = static_cast<unsigned>(ceil_div(M, kRgTokens));
+  hipLaunchKernelGGL((route_gate_kernel<T, G>), dim3(grid), dim3(kGateThreads), 0, st,
+                     static_cast<const T*>(hidden), static_cast<const T*>(gate), M, H, E, topk, renorm, w, ids);
+}
+template <typename T>
+int dispatch_route_gate(const void* hidden, const void* gate, int64_t M, int H, int E, int topk, int renorm,
+                        float* w, int32_t* ids, hipStream_t st) {
+  if (E <= 1) launch_route_gate<T, 1>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
+  else if (E <= 2) launch_route_gate<T, 2>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
+  else if (E <= 4) launch_route_gate<T, 4>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
+  else if (E <= 8) launch_route_gate<T, 8>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
+  else if (E <= 16) launch_route_gate<T, 16>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
+  else if (E <= 32) launch_route_gate<T, 32>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
+  else launch_route_gate<T, 64>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
+  return check_launch("route_gate_kernel");
+}
+}  // namespace
+}  // namespace fr
+
+extern "C" int fr_route_gate(const void* hidden, const void* gate, int dtype, int64_t M, int64_t H, int64_t E,
+                             int topk, int renormalize, float* weights_out, int32_t* ids_out, void* stream) {
+  using namespace fr;
+  FR_REQUIRE(M >= 0, FR_E_SHAPE, "fr_route_gate: M=%lld < 0", (long long)M);
+  if (M == 0) return FR_OK;
+  FR_REQUIRE(hidden && gate && weights_out && ids_out, FR_E_NULL, "fr_route_gate: null pointer");
+  FR_REQUIRE(E >= 1 && E <= kRgMaxE, FR_E_SHAPE, "fr_route_gate: E=%lld outside [1, %d]", (long long)E, kRgMaxE);
+  FR_REQUIRE(topk >= 1 && topk <= E, FR_E_SHAPE, "fr_route_gate: topk=%d outside [1, E=%lld]", topk, (long long)E);
+  FR_REQUIRE(H >= 8 && H % 8 == 0 && H < (int64_t(1) << 30), FR_E_SHAPE, "fr_route_gate: H=%lld must be a multiple of 8", (long long)H);
+  FR_REQUIRE(aligned16(hidden), FR_E_ALIGN, "fr_route_gate: hidden must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == FR_BF16) return dispatch_route_gate<bf16_t>(hidden, gate, M, (int)H, (int)E, topk, renormalize, weights_out, ids_out, st);
+  if (dtype == FR_F16) return dispatch_route_gate<f16_t>(hidden, gate, M, (int)H, (int)E, topk, renormalize, weights_out, ids_out, st);
+  return fail(FR_E_DTYPE, "fr_route_gate: dtype %d not in {f16, bf16}", dtype);
+}

@@ -1,0 +1,285 @@
+// Block-aligned stable counting sort of (expert, token) pairs on gfx950.
+//
+// The n flat pairs are cut into segments of seg_len consecutive pairs, one
+// wavefront per segment.  (1) every wavefront builds an LDS histogram of its
+// segment; (2) an exclusive scan over segments gives each (expert, segment) its
+// offset inside the expert's run, and an exclusive scan over the padded expert
+// totals gives each run its start; (3) every wavefront walks its segment again
+// 64 pairs at a time and ranks the pairs of one expert among themselves with
+// wavefront ballots, so flat order survives inside each expert: the result is
+// the stable sort.  Small inputs run all three phases in one workgroup with the
+// tables in LDS; large ones use three launches and a global table.
+#include "fr_common.h"
+
+namespace fr {
+namespace {
+
+constexpr int kSmallThreads = 1024;
+constexpr int kSmallWaves = kSmallThreads / kWave;
+constexpr int kSmallMaxE = 256;
+constexpr int64_t kSmallMaxN = 16384;
+constexpr int kMaxE = 1024;
+constexpr int kSegThreads = 256;
+constexpr int kSegWaves = kSegThreads / kWave;
+constexpr int kScanThreads = 1024;
+constexpr int kScanWaves = kScanThreads / kWave;
+
+__device__ __forceinline__ int64_t min64(int64_t a, int64_t b) { return a < b ? a : b; }
+
+__host__ __device__ inline int bits_for(int E) {
+  int b = 0;
+  while ((1 << b) < E) ++b;
+  return b;
+}
+
+// lanes (among `valid` ones) holding the same expert as this lane
+__device__ __forceinline__ unsigned long long same_expert_lanes(int e, bool valid, int nbits) {
+  unsigned long long m = __ballot(valid);
+  for (int b = 0; b < nbits; ++b) {
+    const bool bit = (e >> b) & 1;
+    const unsigned long long vote = __ballot(bit);
+    m &= bit ? vote : ~vote;
+  }
+  return m;
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int t = __shfl_up(v, d, kWave);
+    if (lane >= d) v += t;
+  }
+  return v;
+}
+
+template <typename IdT>
+__device__ __forceinline__ void segment_histogram(const IdT* __restrict__ ids, int64_t lo, int64_t hi,
+                                                  int E, int lane, int* hist) {
+  for (int64_t p = lo + lane; p < hi; p += kWave) {
+    const int e = static_cast<int>(ids[p]);
+    if (e >= 0 && e < E) atomicAdd(&hist[e], 1);
+  }
+}
+
+// Walk [lo, hi) in flat order; cnt[e] holds the next free slot of expert e for
+// this wavefront and is advanced as pairs are placed.
+template <typename IdT>
+__device__ __forceinline__ void segment_scatter(const IdT* __restrict__ ids, int64_t lo, int64_t hi,
+                                                int E, int nbits, int lane, volatile int* cnt,
+                                                int32_t* __restrict__ sorted) {
+  const unsigned long long below = (1ull << lane) - 1ull;
+  for (int64_t base = lo; base < hi; base += kWave) {
+    const int64_t p = base + lane;
+    int e = (p < hi) ? static_cast<int>(ids[p]) : 0;
+    const bool valid = (p < hi) && e >= 0 && e < E;
+    if (!valid) e = 0;
+    const unsigned long long same = same_expert_lanes(e, valid, nbits);
+    if (valid) {
+      const int rank = __popcll(same & below);
+      const int total = __popcll(same);
+      const int old = cnt[e];
+      sorted[old + rank] = static_cast<int32_t>(p);
+      if (rank == total - 1) cnt[e] = old + total;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// start[e] = exclusive scan of the padded totals, start[E] = padded length.
+// Executed by one wavefront; total/start live in LDS.
+__device__ __forceinline__ void scan_padded_totals(const int* total, int* start, int E, int B, int lane) {
+  int running = 0;
+  for (int base = 0; base < E; base += kWave) {
+    const int e = base + lane;
+    const int c = (e < E) ? (total[e] + B - 1) / B * B : 0;
+    const int incl = wave_inclusive_scan(c, lane);
+    if (e < E) start[e] = running + incl - c;
+    running += __shfl(incl, kWave - 1, kWave);
+  }
+  if (lane == 0) start[E] = running;
+}
+
+// expert_ids for every block, padding slots of every run, and the tail.
+__device__ __forceinline__ void write_block_table(const int* total, const int* start, int E, int B,
+                                                  int64_t n, int64_t sorted_len, int tid, int nthreads,
+                                                  int32_t* __restrict__ sorted,
+                                                  int32_t* __restrict__ expert_ids,
+                                                  int32_t* __restrict__ npost_out) {
+  const int npost = start[E];
+  const int nblocks = npost / B;
+  for (int b = tid; b < nblocks; b += nthreads) {
+    const int pos = b * B;
+    int lo = 0, hi = E;  // largest e with start[e] <= pos and a non-empty run
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (start[mid] <= pos) lo = mid; else hi = mid;
+    }
+    expert_ids[b] = lo;
+  }
+  const int lane = tid % kWave, wave = tid / kWave, nwaves = nthreads / kWave;
+  for (int e = wave; e < E; e += nwaves) {
+    for (int s = start[e] + total[e] + lane; s < start[e + 1]; s += kWave) sorted[s] = static_cast<int32_t>(n);
+  }
+  for (int64_t s = npost + tid; s < sorted_len; s += nthreads) sorted[s] = static_cast<int32_t>(n);
+  if (tid == 0) npost_out[0] = npost;
+}
+
+// ---------------------------------------------------------------- small path
+template <typename IdT>
+__global__ __launch_bounds__(kSmallThreads) void align_small_kernel(
+    const IdT* __restrict__ ids, int64_t n, int E, int B, int seg_len, int64_t sorted_len,
+    int32_t* __restrict__ sorted, int32_t* __restrict__ expert_ids, int32_t* __restrict__ npost_out) {
+  __shared__ int table[kSmallWaves * kSmallMaxE];
+  __shared__ int total[kSmallMaxE];
+  __shared__ int start[kSmallMaxE + 1];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  for (int i = tid; i < kSmallWaves * E; i += kSmallThreads) table[i] = 0;
+  __syncthreads();
+  const int64_t lo = min64(n, static_cast<int64_t>(wave) * seg_len);
+  const int64_t hi = min64(n, lo + seg_len);
+  segment_histogram(ids, lo, hi, E, lane, &table[wave * E]);
+  __syncthreads();
+  for (int e = tid; e < E; e += kSmallThreads) {
+    int running = 0;
+    for (int w = 0; w < kSmallWaves; ++w) {
+      const int c = table[w * E + e];
+      table[w * E + e] = running;
+      running += c;
+    }
+    total[e] = running;
+  }
+  __syncthreads();
+  if (wave == 0) scan_padded_totals(total, start, E, B, lane);
+  __syncthreads();
+  for (int i = tid; i < kSmallWaves * E; i += kSmallThreads) table[i] += start[i % E];
+  write_block_table(total, start, E, B, n, sorted_len, tid, kSmallThreads, sorted, expert_ids, npost_out);
+  __syncthreads();
+  segment_scatter(ids, lo, hi, E, bits_for(E), lane, &table[wave * E], sorted);
+}
+
+// ---------------------------------------------------------------- large path
+// counts is [E][S]: after align_scan_kernel, counts[e][s] is the offset of
+// segment s inside expert e's run and run_start[e] the start of the run.
+template <typename IdT>
+__global__ __launch_bounds__(kSegThreads) void align_count_kernel(
+    const IdT* __restrict__ ids, int64_t n, int E, int seg_len, int S, int* __restrict__ counts) {
+  extern __shared__ int hist[];  // [kSegWaves][E]
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int seg = blockIdx.x * kSegWaves + wave;
+  int* mine = hist + wave * E;
+  for (int e = lane; e < E; e += kWave) mine[e] = 0;
+  __builtin_amdgcn_wave_barrier();
+  if (seg >= S) return;
+  const int64_t lo = static_cast<int64_t>(seg) * seg_len;
+  const int64_t hi = min64(n, lo + seg_len);
+  segment_histogram(ids, lo, hi, E, lane, mine);
+  __builtin_amdgcn_wave_barrier();
+  for (int e = lane; e < E; e += kWave) counts[static_cast<int64_t>(e) * S + seg] = mine[e];
+}
+
+__global__ __launch_bounds__(kScanThreads) void align_scan_kernel(
+    int* __restrict__ counts, int* __restrict__ run_start, int64_t n, int E, int B, int S,
+    int64_t sorted_len, int32_t* __restrict__ sorted, int32_t* __restrict__ expert_ids,
+    int32_t* __restrict__ npost_out) {
+  __shared__ int total[kMaxE];
+  __shared__ int start[kMaxE + 1];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  for (int e = wave; e < E; e += kScanWaves) {
+    int* row = counts + static_cast<int64_t>(e) * S;
+    int running = 0;
+    for (int base = 0; base < S; base += kWave) {
+      const int s = base + lane;
+      const int c = (s < S) ? row[s] : 0;
+      const int incl = wave_inclusive_scan(c, lane);
+      if (s < S) row[s] = running + incl - c;
+      running += __shfl(incl, kWave - 1, kWave);
+    }
+    if (lane == 0) total[e] = running;
+  }
+  __syncthreads();
+  if (wave == 0) scan_padded_totals(total, start, E, B, lane);
+  __syncthreads();
+  for (int e = tid; e < E; e += kScanThreads) run_start[e] = start[e];
+  write_block_table(total, start, E, B, n, sorted_len, tid, kScanThreads, sorted, expert_ids, npost_out);
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(kSegThreads) void align_scatter_kernel(
+    const IdT* __restrict__ ids, int64_t n, int E, int seg_len, int S, const int* __restrict__ counts,
+    const int* __restrict__ run_start, int32_t* __restrict__ sorted) {
+  extern __shared__ int hist[];  // [kSegWaves][E]
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int seg = blockIdx.x * kSegWaves + wave;
+  if (seg >= S) return;
+  int* mine = hist + wave * E;
+  for (int e = lane; e < E; e += kWave) mine[e] = run_start[e] + counts[static_cast<int64_t>(e) * S + seg];
+  __builtin_amdgcn_wave_barrier();
+  const int64_t lo = static_cast<int64_t>(seg) * seg_len;
+  const int64_t hi = min64(n, lo + seg_len);
+  segment_scatter(ids, lo, hi, E, bits_for(E), lane, mine, sorted);
+}
+
+bool use_small_path(int64_t n, int E) { return n <= kSmallMaxN && E <= kSmallMaxE; }
+
+int large_seg_len(int64_t n) {
+  const int64_t want = round_up(ceil_div(n, 2048), kWave);
+  return static_cast<int>(want < 256 ? 256 : want);
+}
+
+template <typename IdT>
+int run(const void* ids_v, int64_t n, int E, int B, int32_t* sorted, int32_t* expert_ids,
+        int32_t* npost, void* ws, hipStream_t st) {
+  const IdT* ids = static_cast<const IdT*>(ids_v);
+  const int64_t sorted_len = n + static_cast<int64_t>(E) * (B - 1);
+  if (use_small_path(n, E)) {
+    int seg_len = static_cast<int>(round_up(ceil_div(n, kSmallWaves), kWave));
+    if (seg_len == 0) seg_len = kWave;
+    hipLaunchKernelGGL((align_small_kernel<IdT>), dim3(1), dim3(kSmallThreads), 0, st, ids, n, E, B,
+                       seg_len, sorted_len, sorted, expert_ids, npost);
+    return check_launch("align_small_kernel");
+  }
+  const int seg_len = large_seg_len(n);
+  const int S = static_cast<int>(ceil_div(n, seg_len));
+  int* counts = static_cast<int*>(ws);
+  int* run_start = counts + static_cast<int64_t>(E) * S;
+  const unsigned blocks = static_cast<unsigned>(ceil_div(S, kSegWaves));
+  const size_t lds = sizeof(int) * kSegWaves * E;
+  hipLaunchKernelGGL((align_count_kernel<IdT>), dim3(blocks), dim3(kSegThreads), lds, st, ids, n, E,
+                     seg_len, S, counts);
+  hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, counts, run_start, n, E, B, S,
+                     sorted_len, sorted, expert_ids, npost);
+  hipLaunchKernelGGL((align_scatter_kernel<IdT>), dim3(blocks), dim3(kSegThreads), lds, st, ids, n, E,
+                     seg_len, S, counts, run_start, sorted);
+  return check_launch("align kernels");
+}
+
+}  // namespace
+}  // namespace fr
+
+extern "C" int64_t fr_moe_align_workspace_bytes(int64_t n, int E) {
+  using namespace fr;
+  if (n < 0 || E < 1 || E > kMaxE) return -1;
+  if (use_small_path(n, E)) return 0;
+  const int64_t S = ceil_div(n, large_seg_len(n));
+  return static_cast<int64_t>(sizeof(int)) * (static_cast<int64_t>(E) * S + E);
+}
+
+extern "C" int fr_moe_align(const void* topk_ids, int ids_dtype, int64_t n, int E, int block,
+                            int32_t* sorted_token_ids, int32_t* expert_ids,
+                            int32_t* num_tokens_post_pad, void* workspace, int64_t workspace_bytes,
+                            void* stream) {
+  using namespace fr;
+  FR_REQUIRE(n >= 0 && n <= (int64_t(1) << 30), FR_E_SHAPE, "fr_moe_align: n=%lld outside [0, 2^30]", (long long)n);
+  FR_REQUIRE(E >= 1 && E <= kMaxE, FR_E_SHAPE, "fr_moe_align: E=%d outside [1, %d]", E, kMaxE);
+  FR_REQUIRE(block >= 1 && block <= 4096, FR_E_SHAPE, "fr_moe_align: block=%d outside [1, 4096]", block);
+  FR_REQUIRE(n + int64_t(E) * block < (int64_t(1) << 31), FR_E_SHAPE, "fr_moe_align: padded length overflows int32");
+  FR_REQUIRE(sorted_token_ids && expert_ids && num_tokens_post_pad, FR_E_NULL, "fr_moe_align: null output pointer");
+  FR_REQUIRE(n == 0 || topk_ids, FR_E_NULL, "fr_moe_align: null topk_ids");
+  FR_REQUIRE(ids_dtype == FR_I32 || ids_dtype == FR_I64, FR_E_DTYPE, "fr_moe_align: ids dtype %d not in {i32, i64}", ids_dtype);
+  const int64_t need = fr_moe_align_workspace_bytes(n, E);
+  FR_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), FR_E_WORKSPACE,
+             "fr_moe_align: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)need);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (ids_dtype == FR_I32) return run<int32_t>(topk_ids, n, E, block, sorted_token_ids, expert_ids, num_tokens_post_pad, workspace, st);
+  return run<int64_t>(topk_ids, n, E, block, sorted_token_ids, expert_ids, num_tokens_post_pad, workspace, st);
+}

@@ -1,0 +1,148 @@
+/* fast_route_hip.h -- C ABI of the MI355X (gfx950) fused-MoE library.
+ *
+ * Every entry point is what a binding of the reference's hot path calls; the
+ * comment on each names the reference interface it replaces
+ * (hgl71964/fast-route, paths relative to the reference root).
+ *
+ * Conventions
+ *   - all pointers except `stream` are DEVICE addresses owned by the caller;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - every call only enqueues work on `stream`: no allocation, no host
+ *     synchronisation, no device-to-host copy, safe under graph capture;
+ *   - return value 0 on success, a negative FR_E_* code otherwise;
+ *     fr_last_error_string() gives the thread-local message of the last failure;
+ *   - tensors are dense row-major unless a stride argument says otherwise.
+ */
+#ifndef FAST_ROUTE_HIP_H
+#define FAST_ROUTE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FR_OK 0
+#define FR_E_NULL (-1)        /* a required pointer is NULL                     */
+#define FR_E_SHAPE (-2)       /* a dimension is out of the supported range      */
+#define FR_E_DTYPE (-3)       /* dtype enum not supported by this entry point   */
+#define FR_E_ALIGN (-4)       /* pointer / stride not aligned as required       */
+#define FR_E_WORKSPACE (-5)   /* workspace too small                            */
+#define FR_E_LAUNCH (-6)      /* the HIP runtime rejected a launch              */
+#define FR_E_NO_DEVICE (-7)   /* no gfx950 device / code object not loadable    */
+
+typedef enum fr_dtype {
+  FR_F16 = 0,
+  FR_BF16 = 1,
+  FR_F32 = 2,
+  FR_FP8_E4M3 = 3, /* OCP e4m3fn */
+  FR_I32 = 4,
+  FR_I64 = 5
+} fr_dtype;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int fr_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* fr_last_error_string(void);
+
+/* ---- gating --------------------------------------------------------------
+ * Top-k gating of router logits[M, E] (row stride `ld` elements): stable
+ * descending order of the fp32 logits (ties -> lower expert index), softmax
+ * over the selected logits (renormalize != 0) or the selected entries of the
+ * full softmax (renormalize == 0).  Writes weights_out[M, topk] fp32 and
+ * ids_out[M, topk] int32, both contiguous.
+ * Replaces: route_kernel's sort+softmax, fast_route/fast_route/ops/stable_route.py:97-121,
+ * and vLLM topk_softmax + renormalise, fast_route/fast_route/layers/vllm_route.py:79-87.
+ * Limits: 1 <= topk <= E <= 256; logits_dtype in {FR_F16, FR_BF16, FR_F32}. */
+int fr_gating_topk(const void* logits, int logits_dtype, int64_t M, int64_t E, int64_t ld,
+                   int topk, int renormalize, float* weights_out, int32_t* ids_out, void* stream);
+
+/* Gate-matrix form: logits = hidden[M, H] @ gate[H, E] accumulated in fp32,
+ * then fr_gating_topk, in one kernel (no [M, E] round trip).
+ * Replaces: fused_route, fast_route/fast_route/ops/stable_route.py:123-178.
+ * Limits: E <= 64, H % 8 == 0; dtype in {FR_F16, FR_BF16}. */
+int fr_route_gate(const void* hidden, const void* gate, int dtype, int64_t M, int64_t H, int64_t E,
+                  int topk, int renormalize, float* weights_out, int32_t* ids_out, void* stream);
+
+/* ---- routing arrays ------------------------------------------------------
+ * Block-aligned stable counting sort of the n = M*topk flat expert ids.
+ *   sorted_token_ids : int32[n + E*(block-1)], fully written; padding = n
+ *   expert_ids       : int32[n + E], first num_tokens_post_pad/block entries written
+ *   num_tokens_post_pad : int32[1]
+ * Replaces: moe_align_block_size, fast_route/fast_route/ops/fused_moe.py:133-175
+ * (vLLM ops.moe_align_block_size at :173).
+ * ids_dtype in {FR_I32, FR_I64}; 1 <= E <= 1024; block >= 1; ids must lie in [0, E).
+ * `workspace` must hold fr_moe_align_workspace_bytes(n, E) bytes (may be 0). */
+int64_t fr_moe_align_workspace_bytes(int64_t n, int E);
+int fr_moe_align(const void* topk_ids, int ids_dtype, int64_t n, int E, int block,
+                 int32_t* sorted_token_ids, int32_t* expert_ids, int32_t* num_tokens_post_pad,
+                 void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- grouped GEMM, op level ----------------------------------------------
+ * For every sorted slot s < num_tokens_post_pad with p = sorted_token_ids[s] < num_valid:
+ *   C[p, :] = A[p / top_k, :] @ B[expert_ids[s / block], :, :]^T   (fp32 accumulate)
+ * optionally times topk_weights[p], rounded to `dtype`.
+ *   A [*, K] (row stride lda), B [E, N, K] dense, C [num_valid, N] dense.
+ * Replaces: invoke_fused_moe_kernel / fused_moe_kernel,
+ * fast_route/fast_route/ops/fused_moe.py:178-214 and :10-130.
+ * Limits: K % 32 == 0, N % 4 == 0, block in {16, 32, 64, 128}; dtype in {FR_F16, FR_BF16}. */
+int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, void* C,
+                        const float* topk_weights, const int32_t* sorted_token_ids,
+                        const int32_t* expert_ids, const int32_t* num_tokens_post_pad,
+                        int64_t sorted_len, int64_t num_valid, int64_t N, int64_t K, int E,
+                        int block, int top_k, int mul_routed_weight, int dtype, void* stream);
+
+/* ---- fused expert MLPs ---------------------------------------------------
+ * Tile plan chosen from the problem size: the routing block the fused kernels
+ * want (pass it to fr_moe_align) and the split-K factor of the down GEMM. */
+typedef struct fr_moe_plan {
+  int32_t block;      /* routing block = token rows per GEMM tile            */
+  int32_t split_k;    /* K splits of the down projection                     */
+  int64_t sorted_len; /* n + E*(block-1): length of sorted_token_ids         */
+  int64_t workspace_bytes; /* bytes fr_fused_moe / fr_fused_experts need     */
+} fr_moe_plan;
+int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk, int dtype, fr_moe_plan* plan);
+
+/* act[s, :] = silu(x[t] @ W1[e, :F]^T) * (x[t] @ W1[e, F:]^T) for every sorted
+ * slot s < num_tokens_post_pad (t = sorted_token_ids[s] / topk, padding slots
+ * compute on token 0), written at row s of act[sorted_len, F].
+ * Replaces: grouped GEMM 1 + silu_and_mul,
+ * fast_route/fast_route/layers/stable_route.py:85-90. */
+int fr_moe_gateup_silu(const void* x, const void* w1, const int32_t* sorted_token_ids,
+                       const int32_t* expert_ids, const int32_t* num_tokens_post_pad,
+                       int64_t M, int64_t H, int64_t F, int E, int topk, int block, int dtype,
+                       void* act, void* stream);
+
+/* out[m, :] = sum_j topk_weights[m, j] * (act[slot(m, j)] @ W2[e]^T), the
+ * down projection with the routed weight applied in the GEMM epilogue and the
+ * top-k combine.  `partial` is fp32 scratch of split_k * M*topk * H elements.
+ * Replaces: grouped GEMM 2 + torch.sum,
+ * fast_route/fast_route/layers/stable_route.py:92-102. */
+int fr_moe_down_combine(const void* act, const void* w2, const float* topk_weights,
+                        const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                        const int32_t* num_tokens_post_pad, int64_t M, int64_t H, int64_t F, int E,
+                        int topk, int block, int split_k, int dtype, float* partial, void* out,
+                        void* stream);
+
+/* Experts only: routing arrays + both GEMMs + combine, from given top-k
+ * weights/ids (the fused_moe(hidden, w1, w2, topk_weights, topk_ids) shape of
+ * benchmarks/swizzle_moe/v0_moe_fused.py:219-293). */
+int fr_fused_experts(const void* x, const void* w1, const void* w2, const float* topk_weights,
+                     const int32_t* topk_ids, int64_t M, int64_t H, int64_t F, int E, int topk,
+                     int dtype, void* out, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Whole layer from router logits[M, E] (dense, `logits_dtype`):
+ * gating -> routing arrays -> gate/up GEMM + SiLU*mul -> down GEMM + combine.
+ * Replaces: fused_moe, fast_route/fast_route/layers/stable_route.py:10-102 and
+ * fast_route/fast_route/layers/vllm_route.py:17-120.  `out` may alias `x`
+ * (the reference's inplace=True). */
+int fr_fused_moe(const void* x, const void* w1, const void* w2, const void* logits,
+                 int logits_dtype, int64_t M, int64_t H, int64_t F, int E, int topk,
+                 int renormalize, int dtype, void* out, void* workspace, int64_t workspace_bytes,
+                 void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FAST_ROUTE_HIP_H */

@@ -1,0 +1,60 @@
+"""CPU-only: the C-ABI library loads and exports every symbol the header declares."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fast_route_hip.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fr_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_expected_entry_points():
+    names = _declared()
+    for must in ("fr_gating_topk", "fr_moe_align", "fr_moe_grouped_gemm", "fr_moe_gateup_silu",
+                 "fr_moe_down_combine", "fr_fused_moe", "fr_fused_experts", "fr_route_gate"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from fast_route_amd import _native
+    if not os.path.exists(_native.LIB_PATH):
+        pytest.fail("libfast_route_hip.so not built: run `python -m fast_route_amd.build`")
+    handle = ctypes.CDLL(_native.LIB_PATH)
+    for name in _declared():
+        assert hasattr(handle, name), "missing export %s" % name
+    # the ctypes table covers the header exactly
+    assert sorted(_native.SIGNATURES) == _declared()
+
+
+def test_host_only_calls_need_no_gpu():
+    from fast_route_amd import _native
+    lib = _native.lib()
+    assert lib.fr_version() >= 100
+    assert lib.fr_moe_align_workspace_bytes(128, 8) == 0
+    assert lib.fr_moe_align_workspace_bytes(393216, 64) > 0
+    assert lib.fr_moe_align_workspace_bytes(10, 5000) == -1
+    p = _native.FrMoePlan()
+    assert lib.fr_moe_get_plan(64, 4096, 14336, 8, 2, _native.FR_BF16, p) == 0
+    assert p.block in (16, 32, 64, 128) and p.split_k >= 1
+    assert p.sorted_len == 128 + 8 * (p.block - 1) and p.workspace_bytes > 0
+    # argument errors come back as codes + message, never as aborts
+    assert lib.fr_moe_get_plan(64, 4095, 14336, 8, 2, _native.FR_BF16, p) == -2
+    assert b"multiples of 128" in lib.fr_last_error_string()
+    with pytest.raises(AssertionError):
+        _native.check(-2)
+    assert lib.fr_gating_topk(None, _native.FR_F32, 4, 8, 8, 2, 1, None, None, None) == -1
+    assert lib.fr_gating_topk(None, _native.FR_F32, 0, 8, 8, 2, 1, None, None, None) == 0
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+    from fast_route_amd.ops.fused_moe import moe_align_block_size
+    with pytest.raises(AssertionError):
+        moe_align_block_size(torch.zeros(4, 2, dtype=torch.int32), 16, 8)

@@ -1,0 +1,104 @@
+"""GPU parity: gating kernels vs the CPU oracle.  ids bit-exact, weights to 1e-6."""
+import sys
+
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+W_ATOL = 2e-6  # fp32 softmax weights in [0, 1]: a few ulp of expf/divide
+
+
+def _say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+def _run_gating(logits_dev, topk, renorm):
+    from fast_route_amd.ops.stable_route import topk_softmax
+    M = logits_dev.shape[0]
+    w = torch.empty((M, topk), dtype=torch.float32, device="cuda")
+    ids = torch.empty((M, topk), dtype=torch.int32, device="cuda")
+    topk_softmax(w, ids, None, logits_dev, renormalize=renorm)
+    torch.cuda.synchronize()
+    return w.cpu(), ids.cpu()
+
+
+@pytest.mark.parametrize("E,topk", [(8, 2), (16, 4), (64, 6), (1, 1), (3, 2), (5, 5), (24, 3), (100, 7), (256, 8)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("renorm", [True, False])
+def test_gating_parity(native, E, topk, dtype, renorm):
+    for M in (1, 63, 1000):
+        _say(f"gating E={E} k={topk} dtype={dtype} renorm={renorm} M={M}")
+        g = torch.Generator().manual_seed(E * 131 + topk * 7 + M)
+        logits = torch.randn(M, E, generator=g).to(dtype)  # bf16/fp16 rounding creates exact ties
+        w, ids = _run_gating(logits.cuda(), topk, renorm)
+        rw, rid = oracle.gating_topk(logits, topk, renorm)
+        assert torch.equal(ids, rid), "gating ids differ"
+        torch.testing.assert_close(w, rw, atol=W_ATOL, rtol=0)
+
+
+def test_gating_ties_and_special_rows(native):
+    _say("gating special rows")
+    rows = [
+        [0.0] * 8,                                   # all equal -> ids 0..k-1
+        [1.0, 3.0, 3.0, 0.0, 3.0, 1.0, 1.0, -2.0],   # three-way tie
+        [-30.0, -30.0, -30.0, -30.0, -30.0, 30.0, -30.0, -30.0],
+        [5.0, 4.0, 3.0, 2.0, 1.0, 0.0, -1.0, -2.0],
+        [-2.0, -1.0, 0.0, 1.0, 2.0, 3.0, 4.0, 5.0],
+    ]
+    logits = torch.tensor(rows)
+    for k in (1, 2, 4, 8):
+        for renorm in (True, False):
+            w, ids = _run_gating(logits.cuda(), k, renorm)
+            rw, rid = oracle.gating_topk(logits, k, renorm)
+            assert torch.equal(ids, rid)
+            torch.testing.assert_close(w, rw, atol=W_ATOL, rtol=0)
+    w, ids = _run_gating(logits.cuda(), 4, True)
+    assert ids[0].tolist() == [0, 1, 2, 3] and ids[1].tolist() == [1, 2, 4, 0]
+
+
+def test_gating_reference_route_test_recipe(native):
+    """tests/test_route.py:12-77 of the reference: weights vs topk(softmax(h@gate)), atol 1e-2."""
+    for seed in range(3):
+        for m, topk in ((128, 2), (512, 4)):
+            _say(f"route recipe seed={seed} m={m} topk={topk}")
+            torch.manual_seed(seed)
+            h = (torch.randn((m, 4096)) / 10).half()
+            gate = (torch.randn((4096, 16)) / 10).half()
+            from fast_route_amd.ops.stable_route import fused_route
+            tw = torch.empty(m, 16, dtype=torch.float32, device="cuda")
+            ti = torch.empty(m, 16, dtype=torch.int32, device="cuda")
+            w, ids = fused_route(h.cuda(), gate.cuda(), topk, tw, ti, True)
+            torch.cuda.synchronize()
+            score = h.float() @ gate.float()
+            rw, rid = torch.topk(torch.softmax(score, -1), topk)
+            rw = rw / rw.sum(-1, keepdim=True)
+            torch.testing.assert_close(w.cpu(), rw, atol=1e-2, rtol=0)
+            ow, oid = oracle.route_from_gate(h, gate, topk)
+            torch.testing.assert_close(w.cpu(), ow, atol=1e-4, rtol=0)
+            # ids can only differ where fp32 accumulation order flips a near-tie
+            assert (ids.cpu() != oid).float().mean() < 0.01
+
+
+@pytest.mark.parametrize("E,topk,H", [(8, 2, 1024), (64, 6, 2048), (16, 4, 520), (5, 2, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_route_gate_fused_gemm(native, E, topk, H, dtype):
+    from fast_route_amd.ops.stable_route import fused_route
+    for M in (1, 70, 300):
+        _say(f"route_gate E={E} k={topk} H={H} dtype={dtype} M={M}")
+        g = torch.Generator().manual_seed(E + H + M)
+        h = (torch.randn(M, H, generator=g) / 4).to(dtype)
+        gate = (torch.randn(H, E, generator=g) / 4).to(dtype)
+        tw = torch.empty(M, topk, dtype=torch.float32, device="cuda")
+        ti = torch.empty(M, topk, dtype=torch.int32, device="cuda")
+        w, ids = fused_route(h.cuda(), gate.cuda(), topk, tw, ti, True)
+        torch.cuda.synchronize()
+        logits = h.double() @ gate.double()
+        ow, oid = oracle.gating_topk(logits.float(), topk, True)
+        # fp32 MFMA accumulation vs float64 reference: ids may flip only at near-ties
+        flips = (ids.cpu() != oid)
+        assert flips.float().mean() < 0.02
+        ok = ~flips.any(dim=1)
+        torch.testing.assert_close(w.cpu()[ok], ow[ok], atol=1e-4, rtol=0)
