@@ -1,0 +1,241 @@
+"""Benchmark of the fused MoE layer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens M] [--no-sweep] [--no-cpu]
+
+A step is one pass of the whole layer (gating -> routing arrays -> gate/up GEMM
+with SiLU*mul -> down GEMM with routed weight -> top-k combine) over one batch
+of M synthetic tokens of the Mixtral-8x7B shape (H4096, F14336, E8, top-2, bf16).
+Inputs and weights are resident in HBM before the timed region.  Prints ONE JSON
+line: the headline token count (default 4096), the per-stage times measured with
+events on the launch stream, the roofline of the dominant kernel, the token sweep
+and the CPU baseline (the fp32 PyTorch oracle on the host cores, bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+SHAPES = {
+    "mixtral": dict(H=4096, F=14336, E=8, topk=2, zipf=False, sweep=[1, 16, 64, 256, 1024, 4096, 16384]),
+    "fine": dict(H=2048, F=1408, E=64, topk=6, zipf=True, sweep=[1, 32, 128, 512, 2048, 8192]),
+    "small": dict(H=1024, F=3584, E=8, topk=2, zipf=False, sweep=[64]),
+}
+
+
+def layer_flops(M, H, F, topk):
+    return 6.0 * M * topk * H * F
+
+
+def layer_bytes(M, H, F, E, topk, active, bw=2, ba=2):
+    """Algorithmic HBM bytes of one layer pass: active experts' weights once,
+    tokens in, logits, activated intermediate written and read once, output,
+    top-k weights/ids written and read."""
+    return (active * 3 * F * H * bw + M * H * ba + M * E * 4 + 2 * M * topk * F * ba + M * H * ba + 16 * M * topk)
+
+
+class Layer:
+    """Device buffers + staged calls through the C ABI for one (shape, M)."""
+
+    def __init__(self, torch, N, shape, M, w1, w2, seed):
+        self.torch, self.N, self.M = torch, N, M
+        self.H, self.F, self.E, self.topk = shape["H"], shape["F"], shape["E"], shape["topk"]
+        dev = "cuda"
+        g = torch.Generator(device=dev).manual_seed(seed + M)
+        self.x = torch.randn(M, self.H, generator=g, device=dev).to(torch.bfloat16)
+        if shape["zipf"]:
+            r = (torch.randperm(self.E, generator=g, device=dev) + 1).double()
+            pz = r.pow(-1.2)
+            self.logits = (torch.log(pz / pz.sum()).float()[None, :] + torch.randn(M, self.E, generator=g, device=dev))
+        else:
+            self.logits = torch.randn(M, self.E, generator=g, device=dev)
+        self.w1, self.w2 = w1, w2
+        self.plan = N.FrMoePlan()
+        N.check(N.lib().fr_moe_get_plan(M, self.H, self.F, self.E, self.topk, N.FR_BF16, self.plan))
+        p, n = self.plan, M * self.topk
+        self.ws = torch.empty(max(p.workspace_bytes, 256), dtype=torch.uint8, device=dev)
+        self.out = torch.empty(M, self.H, dtype=torch.bfloat16, device=dev)
+        # staged buffers
+        self.tw = torch.empty(n, dtype=torch.float32, device=dev)
+        self.ti = torch.empty(n, dtype=torch.int32, device=dev)
+        self.sorted = torch.empty(p.sorted_len, dtype=torch.int32, device=dev)
+        self.eids = torch.empty(n + self.E, dtype=torch.int32, device=dev)
+        self.npost = torch.empty(1, dtype=torch.int32, device=dev)
+        self.aws_bytes = N.lib().fr_moe_align_workspace_bytes(n, self.E)
+        self.aws = torch.empty(max(self.aws_bytes, 256), dtype=torch.uint8, device=dev)
+        self.act = torch.empty(p.sorted_len, self.F, dtype=torch.bfloat16, device=dev)
+        self.partial = torch.empty(p.split_k * n * self.H, dtype=torch.float32, device=dev)
+        self.stream = torch.cuda.current_stream().cuda_stream
+
+    def fused(self):
+        N = self.N
+        N.check(N.lib().fr_fused_moe(self.x.data_ptr(), self.w1.data_ptr(), self.w2.data_ptr(), self.logits.data_ptr(),
+                                     N.FR_F32, self.M, self.H, self.F, self.E, self.topk, 1, N.FR_BF16,
+                                     self.out.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream))
+
+    def staged(self, events=None):
+        N, lib, p = self.N, self.N.lib(), self.plan
+        rec = (lambda i: events[i].record()) if events else (lambda i: None)
+        rec(0)
+        N.check(lib.fr_gating_topk(self.logits.data_ptr(), N.FR_F32, self.M, self.E, self.E, self.topk, 1,
+                                   self.tw.data_ptr(), self.ti.data_ptr(), self.stream))
+        rec(1)
+        N.check(lib.fr_moe_align(self.ti.data_ptr(), N.FR_I32, self.M * self.topk, self.E, p.block, self.sorted.data_ptr(),
+                                 self.eids.data_ptr(), self.npost.data_ptr(), self.aws.data_ptr(), self.aws_bytes, self.stream))
+        rec(2)
+        N.check(lib.fr_moe_gateup_silu(self.x.data_ptr(), self.w1.data_ptr(), self.sorted.data_ptr(), self.eids.data_ptr(),
+                                       self.npost.data_ptr(), self.M, self.H, self.F, self.E, self.topk, p.block, N.FR_BF16,
+                                       self.act.data_ptr(), self.stream))
+        rec(3)
+        N.check(lib.fr_moe_down_combine(self.act.data_ptr(), self.w2.data_ptr(), self.tw.data_ptr(), self.sorted.data_ptr(),
+                                        self.eids.data_ptr(), self.npost.data_ptr(), self.M, self.H, self.F, self.E,
+                                        self.topk, p.block, p.split_k, N.FR_BF16, self.partial.data_ptr(),
+                                        self.out.data_ptr(), self.stream))
+        rec(4)
+
+    def active_experts(self):
+        return int(self.torch.unique(self.ti).numel())
+
+
+def time_layer(torch, layer, steps, warmup):
+    for _ in range(warmup):
+        layer.fused()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        layer.fused()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # per-stage times: the same kernels launched stage by stage with events on the launch stream
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(steps)]
+    layer.staged()
+    torch.cuda.synchronize()
+    for s in range(steps):
+        layer.staged(evs[s])
+    torch.cuda.synchronize()
+    names = ["route", "moe_align", "moe_1+silu_and_mul", "moe_2+sum"]
+    stage_us = {nm: sum(evs[s][i].elapsed_time(evs[s][i + 1]) for s in range(steps)) * 1e3 / steps
+                for i, nm in enumerate(names)}
+    return wall_ms, stage_us
+
+
+def measure(torch, N, shape, M, w1, w2, steps, warmup, seed):
+    layer = Layer(torch, N, shape, M, w1, w2, seed)
+    wall_ms, stage_us = time_layer(torch, layer, steps, warmup)
+    H, F, E, topk = shape["H"], shape["F"], shape["E"], shape["topk"]
+    active = layer.active_experts()
+    fl, by = layer_flops(M, H, F, topk), layer_bytes(M, H, F, E, topk, active)
+    t = wall_ms * 1e-3
+    t_hbm, t_mfma = by / (PEAK_HBM_GBS * 1e9), fl / (PEAK_BF16_TFLOPS * 1e12)
+    bound = "hbm" if t_hbm >= t_mfma else "mfma"
+    rec = {
+        "tokens": M, "us_per_layer": round(wall_ms * 1e3, 2), "tflops": round(fl / t / 1e12, 3),
+        "gbps": round(by / t / 1e9, 1), "active_experts": active, "bound": bound,
+        "roofline_frac": round(max(t_hbm, t_mfma) / t, 4), "block": layer.plan.block, "split_k": layer.plan.split_k,
+        "stage_us": {k: round(v, 2) for k, v in stage_us.items()},
+        "ref_2mnk_tflops": round(2.0 * M * F * H / t / 1e12, 3),
+    }
+    return rec, layer
+
+
+def kernel_roofline(shape, rec):
+    """Roofline of the dominant kernel (gate/up grouped GEMM + SiLU*mul) from its
+    event-measured average duration."""
+    M, H, F, topk = rec["tokens"], shape["H"], shape["F"], shape["topk"]
+    dur = rec["stage_us"]["moe_1+silu_and_mul"] * 1e-6
+    flops = 4.0 * M * topk * H * F
+    byts = rec["active_experts"] * 2 * F * H * 2 + M * H * 2 + M * topk * F * 2
+    if flops / (PEAK_BF16_TFLOPS * 1e12) >= byts / (PEAK_HBM_GBS * 1e9):
+        ach = flops / dur / 1e12
+        return {"kernel": "moe_gemm_kernel<EPI_SILU>", "bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "avg_launch_us": round(dur * 1e6, 2), "algorithmic_flops_per_launch": flops}
+    ach = byts / dur / 1e9
+    return {"kernel": "moe_gemm_kernel<EPI_SILU>", "bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
+            "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+            "avg_launch_us": round(dur * 1e6, 2), "algorithmic_bytes_per_launch": byts}
+
+
+def cpu_baseline(torch, shape, layer, sample_tokens):
+    """fp32 PyTorch oracle on the host cores over the first `sample_tokens` tokens of the same batch."""
+    import oracle
+    m = min(sample_tokens, layer.M)
+    x, logits = layer.x[:m].cpu(), layer.logits[:m].cpu()
+    w1, w2 = layer.w1.cpu(), layer.w2.cpu()
+    t0 = time.perf_counter()
+    ref = oracle.fused_moe(x, w1, w2, logits, shape["topk"], True)
+    dt = time.perf_counter() - t0
+    got = layer.out[:m].float().cpu()
+    err = (got - ref).abs().max().item()
+    return {"value": round(layer_flops(m, shape["H"], shape["F"], shape["topk"]) / dt / 1e12, 4), "unit": "TFLOP/s",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "fp32 PyTorch oracle, first %d tokens of the M=%d batch, weights upcast per expert, 1 rep, %.1f s"
+                      % (m, layer.M, dt),
+            "us_per_layer_sample": round(dt * 1e6, 0), "max_abs_err_vs_gpu": err,
+            "ref_max_abs": ref.abs().max().item()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--tokens", type=int, default=4096, help="headline token count")
+    ap.add_argument("--shape", default="mixtral", choices=sorted(SHAPES))
+    ap.add_argument("--seed", type=int, default=1337)
+    ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-tokens", type=int, default=1024)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build is single-GPU (one MI355X runs the whole layer); --gpus must be 1")
+
+    import torch
+    from fast_route_amd import _native as N
+    N.lib()
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    torch.cuda.set_device(0)
+    shape = SHAPES[args.shape]
+    H, F, E, topk = shape["H"], shape["F"], shape["E"], shape["topk"]
+    g = torch.Generator(device="cuda").manual_seed(args.seed)
+    w1 = (torch.randn(E, 2 * F, H, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    w2 = (torch.randn(E, H, F, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+
+    head, layer = measure(torch, N, shape, args.tokens, w1, w2, args.steps, args.warmup, args.seed)
+    sweep = []
+    if not args.no_sweep:
+        for M in shape["sweep"]:
+            if M == args.tokens:
+                sweep.append(head)
+                continue
+            rec, _ = measure(torch, N, shape, M, w1, w2, args.steps, args.warmup, args.seed)
+            sweep.append(rec)
+    result = {
+        "metric": "moe_layer_tflops_%s_bf16_M%d" % (args.shape, args.tokens),
+        "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(head["us_per_layer"] / 1e3, 4), "us_per_layer": head["us_per_layer"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "%s-shape MoE layer: H=%d F=%d E=%d top-%d, M=%d tokens, bf16 in / fp32 accumulate"
+                               % (args.shape, H, F, E, topk, args.tokens),
+                   "tokens": args.tokens, "hidden": H, "ffn": F, "experts": E, "topk": topk, "seed": args.seed,
+                   "flops_formula": "6*M*topk*H*F"},
+        "layer_roofline_frac": head["roofline_frac"], "layer_bound": head["bound"],
+        "stage_us": head["stage_us"],
+        "roofline": kernel_roofline(shape, head),
+        "sweep": sweep,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, shape, layer, args.cpu_tokens)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

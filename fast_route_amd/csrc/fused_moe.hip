@@ -66,13 +66,14 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   if (avg <= 8) block = 16;
   else if (avg <= 24) block = 32;
   else if (avg <= 64) block = 64;
-  else block = 128;
+  else if (avg <= 384) block = 128;
+  else block = 256;
   // down projection: few feature tiles (N = H), so split K until the grid covers the chip
   const int bf = block >= 64 ? 256 : 128;
   const int64_t active_blocks = n < E ? n : (block >= 64 ? ceil_div(n, block) + E / 2 : E);
   const int64_t tiles = active_blocks * ceil_div(H, bf);
   int split = 1;
-  const int bk = block >= 64 ? 64 : 128;
+  const int bk = 64;
   while (split < 16 && tiles * split < 1024 && F / (split * 2) >= 4 * bk) split *= 2;
   plan->block = block;
   plan->split_k = split;

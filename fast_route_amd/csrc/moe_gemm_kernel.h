@@ -1,0 +1,524 @@
+// Grouped expert GEMM kernel template for gfx950 MFMA.
+//
+// One workgroup computes a tile of BT sorted slots (one routing block, hence
+// one expert) by BF output features.  Both operands are K-contiguous in HBM
+// (tokens [*, K], weights [E, N, K]); tiles of BK are staged through LDS in
+// 16-byte chunks under an XOR swizzle and fed to v_mfma with the WEIGHT rows as
+// the MFMA "A" operand and the TOKEN rows as "B", so a lane's accumulator
+// registers hold 4 consecutive output features of one token and the epilogue
+// stores 8/16-byte vectors.  Three epilogues:
+//   EPI_PLAIN  C[pair] = acc (* routed weight), scattered by sorted id
+//   EPI_SILU   W tile = BF/2 gate rows + the matching BF/2 up rows; writes
+//              silu(gate)*up at the slot's own row of act[sorted_len, F]
+//   EPI_DOWN   partial[split][pair] = acc * routed weight in fp32 (split-K slices)
+// Workgroup ids are first regrouped so that each XCD (ids congruent mod 8) gets
+// a contiguous range of tiles, then walked in groups of GROUP_T token blocks x
+// all feature tiles so co-resident workgroups share weight tiles in their L2.
+#pragma once
+#include "fr_common.h"
+
+#include <type_traits>
+
+namespace fr {
+
+enum { EPI_PLAIN = 0, EPI_SILU = 1, EPI_DOWN = 2 };
+
+struct GemmArgs {
+  const void* X;        // token rows [*, K]
+  int64_t ldx;          // row stride of X in elements
+  const void* W;        // [E, w_rows, K]
+  int64_t w_expert_stride;
+  int64_t ldw;          // row stride of W in elements
+  void* out;
+  int64_t ldo;          // row stride of out in elements
+  int64_t split_stride; // EPI_DOWN: elements between split-K slices
+  const int32_t* sorted;
+  const int32_t* expert_ids;
+  const int32_t* npost;
+  const float* topk_w;  // flat [num_valid] or nullptr
+  int num_valid;        // n = M*topk
+  int top_k;            // X row = sorted id / top_k; 0 => X row = slot index
+  int N;                // output features (EPI_SILU: F, W has 2F rows)
+  int K;
+  int k_per_split;      // multiple of BK
+  int num_t_blocks;     // upper bound on routing blocks
+  int num_f_tiles;
+  int group_t;
+  int mul_weight;
+};
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mfma;
+template <> struct Mfma<bf16_t> {
+  typedef bf16x8 vec8;
+  typedef bf16x4 vec4;
+  static __device__ __forceinline__ f32x16 m32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma<f16_t> {
+  typedef f16x8 vec8;
+  typedef f16x4 vec4;
+  static __device__ __forceinline__ f32x16 m32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+__device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); }
+
+// Tile configuration.  TILE = 32 uses v_mfma_f32_32x32x16, TILE = 16 v_mfma_f32_16x16x32.
+// WT x WF wavefronts split the BT x BF tile; MINB = workgroups per CU the register
+// allocation should allow.  STAGES == 0: tiles go HBM -> registers -> LDS with two
+// LDS buffers (one tile in flight).  STAGES >= 2: tiles go HBM -> LDS directly
+// (global_load_lds_dwordx4) through a ring of STAGES buffers that is refilled as soon
+// as a tile's last fragments are in registers, so STAGES tiles are in flight or landed.
+template <int BT_, int BF_, int BK_, int WT_, int WF_, int TILE_, int MINB_ = 1, int STAGES_ = 0>
+struct Cfg {
+  static constexpr int BT = BT_, BF = BF_, BK = BK_, WT = WT_, WF = WF_, TILE = TILE_, MINB = MINB_;
+  static constexpr int STAGES = STAGES_;
+  static constexpr int NBUF = STAGES_ == 0 ? 2 : STAGES_;
+  static constexpr int NT = WT * WF * kWave;       // threads
+  static constexpr int TT = BT / WT, TF = BF / WF; // per-wave tile
+  static constexpr int IT = TT / TILE, JF = TF / TILE;
+  static constexpr int CPR = BK / 8;               // 16-byte chunks per row
+  static constexpr int KSTEP = (TILE == 32) ? 16 : 32;
+  static constexpr int KGROUPS = 64 / TILE;        // lane groups along K in one MFMA
+  static constexpr int XCH = BT * CPR, WCH = BF * CPR;
+  static constexpr int XL = (XCH + NT - 1) / NT, WL = (WCH + NT - 1) / NT;
+  static constexpr int LDS_BYTES = NBUF * (BT + BF) * BK * 2;
+  static constexpr int NW = NT / kWave;
+  static constexpr int XI = XCH / (kWave * NW), WI = WCH / (kWave * NW);  // direct-to-LDS loads per wave per tile
+  static_assert(STAGES_ == 0 || (STAGES_ >= 2 && XCH % (kWave * NW) == 0 && WCH % (kWave * NW) == 0), "direct-to-LDS tiles must split evenly over the wavefronts");
+  static_assert(TT % TILE == 0 && TF % TILE == 0, "wave tile must be a multiple of the MFMA tile");
+  static_assert(NT % CPR == 0, "threads must cover whole rows");
+  static_assert(BK % KSTEP == 0, "BK must be a multiple of the MFMA K");
+};
+
+// LDS is 64 banks x 4 B: a 16-lane phase of ds_read_b128 is conflict-free when its
+// 16 rows land on 16 different 16-byte columns of a 256-byte line.  Rows shorter
+// than a line share it (16/CPR rows per line), so the XOR key is the line index.
+template <int CPR>
+__device__ __forceinline__ int swizzle(int row, int chunk) {
+  constexpr int ROWS_PER_LINE = CPR >= 16 ? 1 : 16 / CPR;
+  constexpr int MASK = CPR >= 16 ? 15 : CPR - 1;
+  return chunk ^ ((row / ROWS_PER_LINE) & MASK);
+}
+
+template <typename T, typename C, int EPI>
+__global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs a) {
+  typedef typename Mfma<T>::vec8 vec8;
+  typedef typename Mfma<T>::vec4 vec4;
+  typedef typename std::conditional<C::TILE == 32, f32x16, f32x4>::type acc_t;
+  constexpr int BT = C::BT, BF = C::BF, BK = C::BK, CPR = C::CPR, NT = C::NT;
+  constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
+  static_assert(EPI != EPI_SILU || C::JF % 2 == 0, "gate and up tiles must pair up inside a wave");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  u32x4* lds = reinterpret_cast<u32x4*>(lds_raw);
+  // buffer b: X tile at b*BUF, W tile right after it
+  constexpr int BUF = C::XCH + C::WCH;
+
+  // ---- tile coordinates ---------------------------------------------------
+  // The grid is sized for the worst-case padded length; only the first
+  // (npost/BT)*num_f_tiles workgroups have a tile.  Tiles are dealt to the 8 XCDs
+  // (workgroup id mod 8) in contiguous, equally sized ranges of the REAL tile count.
+  const int npost = a.npost[0];
+  const int nt = min(npost / BT, a.num_t_blocks);
+  const int total = nt * a.num_f_tiles;
+  if (static_cast<int>(blockIdx.x) >= total) return;
+  int lin;
+  {
+    const int pid = blockIdx.x, xcd = pid & 7, idx = pid >> 3;
+    const int per = total >> 3, rem = total & 7;
+    lin = xcd * per + (xcd < rem ? xcd : rem) + idx;
+  }
+  const int in_group = a.group_t * a.num_f_tiles;
+  const int group_id = lin / in_group;
+  const int first_t = group_id * a.group_t;
+  const int gsz = min(nt - first_t, a.group_t);
+  const int pid_t = first_t + (lin % in_group) % gsz;
+  const int pid_f = (lin % in_group) / gsz;
+  const int expert = a.expert_ids[pid_t];
+  const int split = blockIdx.y;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wt = wave / C::WF, wf = wave % C::WF;
+
+  // ---- global source pointers for this thread's chunks ----------------------
+  const T* X = static_cast<const T*>(a.X);
+  const T* W = static_cast<const T*>(a.W) + static_cast<int64_t>(expert) * a.w_expert_stride;
+  const int k0 = split * a.k_per_split;
+  const int k_tiles = min(a.k_per_split, a.K - k0) / BK;
+  const int chunk = tid % CPR;
+  const int row0 = tid / CPR;
+  constexpr int ROWS_PER_PASS = NT / CPR;
+  constexpr bool X_FULL = (C::XCH % NT == 0), W_FULL = (C::WCH % NT == 0);
+
+  // X row of a tile row (gathered through the routing arrays) and W row of a tile row
+  auto x_src_row = [&](int rr) -> int64_t {
+    if (a.top_k > 0) {
+      const int sid = a.sorted[pid_t * BT + rr];
+      return sid < a.num_valid ? sid / a.top_k : 0;
+    }
+    return static_cast<int64_t>(pid_t) * BT + rr;
+  };
+  auto w_src_row = [&](int rr) -> int {
+    if constexpr (EPI == EPI_SILU) {
+      const int half = rr / (BF / 2), f = pid_f * (BF / 2) + rr % (BF / 2);
+      return half * a.N + (f < a.N ? f : a.N - 1);
+    } else {
+      const int f = pid_f * BF + rr;
+      return f < a.N ? f : a.N - 1;
+    }
+  };
+
+  // ---- per-lane fragment rows ---------------------------------------------
+  const int frow = lane % C::TILE;  // row inside an MFMA tile
+  const int kgrp = lane / C::TILE;  // which 8-element K group of the MFMA this lane feeds
+  int xoff[C::IT], woff[C::JF];     // chunk offset of the lane's row, swizzle key folded in below
+  int xkey[C::IT], wkey[C::JF];
+#pragma unroll
+  for (int i = 0; i < C::IT; ++i) {
+    const int r = wt * C::TT + i * C::TILE + frow;
+    xoff[i] = r * CPR;
+    xkey[i] = swizzle<CPR>(r, 0);
+  }
+#pragma unroll
+  for (int j = 0; j < C::JF; ++j) {
+    int base;
+    if constexpr (EPI == EPI_SILU) {
+      constexpr int HJ = C::JF / 2;  // first half of the wave's tiles: gate, second: up
+      base = (j < HJ) ? wf * (C::TF / 2) + j * C::TILE : BF / 2 + wf * (C::TF / 2) + (j - HJ) * C::TILE;
+    } else {
+      base = wf * C::TF + j * C::TILE;
+    }
+    const int r = base + frow;
+    woff[j] = C::XCH + r * CPR;
+    wkey[j] = swizzle<CPR>(r, 0);
+  }
+
+  acc_t acc[C::JF][C::IT];
+#pragma unroll
+  for (int j = 0; j < C::JF; ++j)
+#pragma unroll
+    for (int i = 0; i < C::IT; ++i)
+#pragma unroll
+      for (int r = 0; r < ACC_N; ++r) acc[j][i][r] = 0.f;
+
+#define FR_COMPUTE_TILE(buf)                                                          \
+  {                                                                                   \
+    const u32x4* tile = lds + (buf) * BUF;                                            \
+    _Pragma("unroll") for (int ks = 0; ks < BK / C::KSTEP; ++ks) {                    \
+      const int kc = ks * C::KGROUPS + kgrp;                                          \
+      vec8 xf[C::IT], wfr[C::JF];                                                     \
+      _Pragma("unroll") for (int i = 0; i < C::IT; ++i) {                             \
+        const u32x4 v = tile[xoff[i] + (kc ^ xkey[i])];                               \
+        xf[i] = __builtin_bit_cast(vec8, v);                                          \
+      }                                                                               \
+      _Pragma("unroll") for (int j = 0; j < C::JF; ++j) {                             \
+        const u32x4 v = tile[woff[j] + (kc ^ wkey[j])];                               \
+        wfr[j] = __builtin_bit_cast(vec8, v);                                         \
+      }                                                                               \
+      _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                               \
+        _Pragma("unroll") for (int i = 0; i < C::IT; ++i) {                           \
+          if constexpr (C::TILE == 32) acc[j][i] = Mfma<T>::m32(wfr[j], xf[i], acc[j][i]); \
+          else acc[j][i] = Mfma<T>::m16(wfr[j], xf[i], acc[j][i]);                    \
+        }                                                                             \
+    }                                                                                 \
+  }
+
+
+  if constexpr (C::STAGES == 0) {
+  const T* xsrc[C::XL];
+  int xdst[C::XL];
+#pragma unroll
+  for (int i = 0; i < C::XL; ++i) {
+    const int r = row0 + i * ROWS_PER_PASS;
+    const int rr = r < BT ? r : BT - 1;
+    xsrc[i] = X + x_src_row(rr) * a.ldx + k0 + chunk * 8;
+    xdst[i] = rr * CPR + swizzle<CPR>(rr, chunk);
+  }
+  const T* wsrc[C::WL];
+  int wdst[C::WL];
+#pragma unroll
+  for (int i = 0; i < C::WL; ++i) {
+    const int r = row0 + i * ROWS_PER_PASS;
+    const int rr = r < BF ? r : BF - 1;
+    wsrc[i] = W + static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + chunk * 8;
+    wdst[i] = C::XCH + rr * CPR + swizzle<CPR>(rr, chunk);
+  }
+
+  u32x4 xreg[C::XL], wreg[C::WL];
+
+#define FR_LOAD_TILE(kt)                                                              \
+  {                                                                                   \
+    _Pragma("unroll") for (int i = 0; i < C::XL; ++i)                                 \
+      if (X_FULL || row0 + i * ROWS_PER_PASS < BT)                                    \
+        xreg[i] = *reinterpret_cast<const u32x4*>(xsrc[i] + (kt) * BK);               \
+    _Pragma("unroll") for (int i = 0; i < C::WL; ++i)                                 \
+      if (W_FULL || row0 + i * ROWS_PER_PASS < BF)                                    \
+        wreg[i] = *reinterpret_cast<const u32x4*>(wsrc[i] + (kt) * BK);               \
+  }
+#define FR_STORE_TILE(buf)                                                            \
+  {                                                                                   \
+    _Pragma("unroll") for (int i = 0; i < C::XL; ++i)                                 \
+      if (X_FULL || row0 + i * ROWS_PER_PASS < BT) lds[(buf) * BUF + xdst[i]] = xreg[i]; \
+    _Pragma("unroll") for (int i = 0; i < C::WL; ++i)                                 \
+      if (W_FULL || row0 + i * ROWS_PER_PASS < BF) lds[(buf) * BUF + wdst[i]] = wreg[i]; \
+  }
+  // ---- main loop: register-staged double buffering, last tile peeled ---------
+  FR_LOAD_TILE(0);
+  FR_STORE_TILE(0);
+  __syncthreads();
+  for (int kt = 0; kt < k_tiles - 1; ++kt) {
+    const int buf = kt & 1;
+    FR_LOAD_TILE(kt + 1);
+    __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the MFMA block
+    FR_COMPUTE_TILE(buf);
+    __builtin_amdgcn_sched_barrier(0);
+    FR_STORE_TILE(buf ^ 1);
+    __syncthreads();
+  }
+  FR_COMPUTE_TILE((k_tiles - 1) & 1);
+#undef FR_LOAD_TILE
+#undef FR_STORE_TILE
+
+  } else {
+    // ---- direct-to-LDS ring --------------------------------------------------
+    // A wavefront-wide global_load_lds_dwordx4 fills 64 consecutive 16-byte LDS
+    // slots (slot = row*CPR + physical chunk), lane L the L-th of them, so each
+    // lane fetches the logical chunk that the swizzle maps to its slot.
+    typedef const __attribute__((address_space(1))) void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI;
+#ifdef FR_TUNE_XI
+    constexpr int LPT = FR_TUNE_XI + FR_TUNE_WI;
+#else
+    constexpr int LPT = XI + WI;
+#endif
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const T* xsrc[XI];
+    const T* wsrc[WI];
+#pragma unroll
+    for (int i = 0; i < XI; ++i) {
+      const int slot = (i * NW + wave_u) * kWave + lane;
+      const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
+      xsrc[i] = X + x_src_row(rr) * a.ldx + k0 + c * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < WI; ++i) {
+      const int slot = (i * NW + wave_u) * kWave + lane;
+      const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
+      wsrc[i] = W + static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * 8;
+    }
+#ifndef FR_TUNE_XI
+#define FR_TUNE_XI XI
+#define FR_TUNE_WI WI
+#endif
+#define FR_ISSUE_TILE(kt, stage)                                                                    \
+  {                                                                                                 \
+    unsigned char* sbase = lds_raw + (stage) * (BUF * 16);                                          \
+    _Pragma("unroll") for (int i = 0; i < FR_TUNE_XI; ++i)                                          \
+      __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[i] + (kt) * BK),                               \
+                                       (lptr_t)(sbase + (i * NW + wave_u) * (kWave * 16)), 16, 0, 0); \
+    _Pragma("unroll") for (int i = 0; i < FR_TUNE_WI; ++i)                                          \
+      __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + (kt) * BK),                               \
+                                       (lptr_t)(sbase + C::XCH * 16 + (i * NW + wave_u) * (kWave * 16)), 16, 0, 0); \
+  }
+    // wait until at most `tiles_after` later tiles of this lane's loads are still in flight
+    auto wait_tiles = [&](int tiles_after) {
+      if (S > 4 && tiles_after >= 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S > 4 ? 4 * LPT : 0) : "memory");
+      else if (S > 3 && tiles_after == 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S > 3 ? 3 * LPT : 0) : "memory");
+      else if (S > 2 && tiles_after == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S > 2 ? 2 * LPT : 0) : "memory");
+      else if (tiles_after == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+    static_assert(S <= 5 && (S - 1) * LPT <= 63, "vmcnt budget");
+    // Software pipeline: fragments are double-buffered in registers; while the
+    // MFMAs of K-step ks run, the ds_reads of K-step ks+1 are in flight.  The
+    // barrier that publishes tile kt+1 sits before the LAST K-step of tile kt,
+    // whose fragments are already in registers, so no wavefront waits on LDS
+    // latency right after a barrier.
+    constexpr int KS = BK / C::KSTEP;
+    static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
+    vec8 xf[2][C::IT], wfr[2][C::JF];
+#ifdef FR_TUNE_NO_READ
+#define FR_READ_FRAGS(stage_, ks_, fb_) { if ((ks_) == 100) { xf[fb_][0] = __builtin_bit_cast(vec8, lds[stage_]); } }
+#else
+#define FR_READ_FRAGS(stage_, ks_, fb_)                                                 \
+  {                                                                                     \
+    const u32x4* tile = lds + (stage_) * BUF;                                           \
+    const int kc = (ks_) * C::KGROUPS + kgrp;                                           \
+    _Pragma("unroll") for (int i = 0; i < C::IT; ++i)                                   \
+      xf[fb_][i] = __builtin_bit_cast(vec8, tile[xoff[i] + (kc ^ xkey[i])]);            \
+    _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                                   \
+      wfr[fb_][j] = __builtin_bit_cast(vec8, tile[woff[j] + (kc ^ wkey[j])]);           \
+  }
+#endif
+#ifdef FR_TUNE_NO_MMA  /* bottleneck bisection builds only: one MFMA per call keeps the fragments live */
+#define FR_MMA(fb_, j0_, j1_)                                                           \
+  {                                                                                     \
+    if ((j0_) == 0) { _Pragma("unroll") for (int i = 0; i < C::IT; ++i) _Pragma("unroll") for (int j = 0; j < C::JF; ++j) { acc[j][i][0] += __builtin_bit_cast(f32x4, xf[fb_][i])[0] + __builtin_bit_cast(f32x4, wfr[fb_][j])[0]; } } \
+  }
+#else
+#define FR_MMA(fb_, j0_, j1_)                                                           \
+  {                                                                                     \
+    _Pragma("unroll") for (int j = (j0_); j < (j1_); ++j)                               \
+      _Pragma("unroll") for (int i = 0; i < C::IT; ++i) {                               \
+        if constexpr (C::TILE == 32) acc[j][i] = Mfma<T>::m32(wfr[fb_][j], xf[fb_][i], acc[j][i]); \
+        else acc[j][i] = Mfma<T>::m16(wfr[fb_][j], xf[fb_][i], acc[j][i]);              \
+      }                                                                                 \
+  }
+#endif
+    // One K-step: first MFMAs of the step, then the ds_reads of the NEXT step (other
+    // fragment buffer), then the remaining MFMAs, which cover the LDS latency.
+    constexpr int JSPLIT = (C::JF + 1) / 2;
+#define FR_KSTEP(fb_, READ_NEXT)                 \
+  {                                              \
+    __builtin_amdgcn_sched_barrier(0);           \
+    FR_MMA(fb_, 0, JSPLIT);                      \
+    __builtin_amdgcn_sched_barrier(0);           \
+    READ_NEXT;                                   \
+    __builtin_amdgcn_sched_barrier(0);           \
+    FR_MMA(fb_, JSPLIT, C::JF);                  \
+    __builtin_amdgcn_sched_barrier(0);           \
+  }
+#pragma unroll
+    for (int t = 0; t < S; ++t)
+      if (t < k_tiles) FR_ISSUE_TILE(t, t);
+    wait_tiles(min(S - 1, k_tiles - 1));
+    __builtin_amdgcn_s_barrier();
+    FR_READ_FRAGS(0, 0, 0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): no scalar load may be pending when the loop starts
+    int stage = 0;  // ring slot of tile kt
+    // steady state: tile kt+S exists, so the body is one basic block with a fixed
+    // vmcnt and the compiler can count the outstanding LDS reads exactly
+    int kt = 0;
+    for (; kt < k_tiles - S; ++kt) {
+      const int next = (stage + 1 == S) ? 0 : stage + 1;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + 1 < KS) {
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(stage, ks + 1, (ks + 1) & 1));
+        } else {
+          // tile kt+1 landed (this lane's part) and this wavefront's reads of tile kt are done
+          asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((S - 2) * LPT) : "memory");
+          __builtin_amdgcn_s_barrier();  // ... everyone's: slot `stage` can be refilled
+          FR_ISSUE_TILE(kt + S, stage);
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(next, 0, 0));
+        }
+      }
+      stage = next;
+    }
+    // drain: every remaining tile is already in flight, nothing left to issue
+    for (; kt < k_tiles - 1; ++kt) {
+      const int next = (stage + 1 == S) ? 0 : stage + 1;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + 1 < KS) {
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(stage, ks + 1, (ks + 1) & 1));
+        } else {
+          wait_tiles(k_tiles - 2 - kt);
+          __builtin_amdgcn_s_barrier();
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(next, 0, 0));
+        }
+      }
+      stage = next;
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {  // last tile
+      if (ks + 1 < KS) {
+        FR_KSTEP(ks & 1, FR_READ_FRAGS(stage, ks + 1, (ks + 1) & 1));
+      } else {
+        FR_KSTEP(ks & 1, {});
+      }
+    }
+#undef FR_READ_FRAGS
+#undef FR_MMA
+#undef FR_KSTEP
+#undef FR_ISSUE_TILE
+  }
+#undef FR_COMPUTE_TILE
+
+  // ---- epilogue -------------------------------------------------------------
+  // lane holds token column (lane % TILE) of each token tile and, per accumulator
+  // group g (TILE==32: 4 groups of 4 regs; TILE==16: one), 4 consecutive features
+  // starting at g*8 + kgrp*4 (TILE==32) or kgrp*4 (TILE==16) inside the MFMA tile.
+  constexpr int GROUPS = ACC_N / 4;
+#pragma unroll
+  for (int i = 0; i < C::IT; ++i) {
+    const int slot = pid_t * BT + wt * C::TT + i * C::TILE + frow;
+    if constexpr (EPI == EPI_SILU) {
+      constexpr int HJ = C::JF / 2;
+      T* orow = static_cast<T*>(a.out) + static_cast<int64_t>(slot) * a.ldo;
+#pragma unroll
+      for (int j = 0; j < HJ; ++j)
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+          const int f = pid_f * (BF / 2) + wf * (C::TF / 2) + j * C::TILE + g * 8 + kgrp * 4;
+          vec4 o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            o[r] = static_cast<T>(silu(acc[j][i][g * 4 + r]) * acc[j + HJ][i][g * 4 + r]);
+          if (f + 3 < a.N) *reinterpret_cast<vec4*>(orow + f) = o;
+          else
+            for (int r = 0; r < 4; ++r)
+              if (f + r < a.N) orow[f + r] = o[r];
+        }
+    } else {
+      const int sid = a.sorted[slot];
+      if (sid < a.num_valid) {
+        const float rw = a.mul_weight ? a.topk_w[sid] : 1.f;
+#pragma unroll
+        for (int j = 0; j < C::JF; ++j)
+#pragma unroll
+          for (int g = 0; g < GROUPS; ++g) {
+            const int f = pid_f * BF + wf * C::TF + j * C::TILE + g * 8 + kgrp * 4;
+            if constexpr (EPI == EPI_DOWN) {
+              float* orow = static_cast<float*>(a.out) + static_cast<int64_t>(split) * a.split_stride +
+                            static_cast<int64_t>(sid) * a.ldo;
+              f32x4 o;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) o[r] = acc[j][i][g * 4 + r] * rw;
+              if (f + 3 < a.N) *reinterpret_cast<f32x4*>(orow + f) = o;
+              else
+                for (int r = 0; r < 4; ++r)
+                  if (f + r < a.N) orow[f + r] = o[r];
+            } else {
+              T* orow = static_cast<T*>(a.out) + static_cast<int64_t>(sid) * a.ldo;
+              vec4 o;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) o[r] = static_cast<T>(acc[j][i][g * 4 + r] * rw);
+              if (f + 3 < a.N) *reinterpret_cast<vec4*>(orow + f) = o;
+              else
+                for (int r = 0; r < 4; ++r)
+                  if (f + r < a.N) orow[f + r] = o[r];
+            }
+          }
+      }
+    }
+  }
+}
+
+template <typename T, typename C, int EPI>
+int launch_gemm(const GemmArgs& a, int splits, hipStream_t st) {
+  static bool attr_set = false;
+  if (C::LDS_BYTES > 65536 && !attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_kernel<T, C, EPI>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if (e != hipSuccess) return fail(FR_E_LAUNCH, "hipFuncSetAttribute(%d B LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
+    attr_set = true;
+  }
+  const unsigned grid_x = static_cast<unsigned>(a.num_t_blocks) * static_cast<unsigned>(a.num_f_tiles);
+  hipLaunchKernelGGL((moe_gemm_kernel<T, C, EPI>), dim3(grid_x, splits), dim3(C::NT), C::LDS_BYTES, st, a);
+  return check_launch("moe_gemm_kernel");
+}
+
+}  // namespace fr

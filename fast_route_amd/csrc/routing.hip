@@ -239,7 +239,7 @@ int run(const void* ids_v, int64_t n, int E, int B, int32_t* sorted, int32_t* ex
     return check_launch("align_small_kernel");
   }
   const int seg_len = large_seg_len(n);
-  const int S = static_cast<int>(ceil_div(n, seg_len));
+  const int S = static_cast<int>(n > 0 ? ceil_div(n, seg_len) : 1);
   int* counts = static_cast<int*>(ws);
   int* run_start = counts + static_cast<int64_t>(E) * S;
   const unsigned blocks = static_cast<unsigned>(ceil_div(S, kSegWaves));
@@ -260,7 +260,7 @@ extern "C" int64_t fr_moe_align_workspace_bytes(int64_t n, int E) {
   using namespace fr;
   if (n < 0 || E < 1 || E > kMaxE) return -1;
   if (use_small_path(n, E)) return 0;
-  const int64_t S = ceil_div(n, large_seg_len(n));
+  const int64_t S = n > 0 ? ceil_div(n, large_seg_len(n)) : 1;
   return static_cast<int64_t>(sizeof(int)) * (static_cast<int64_t>(E) * S + E);
 }
 
@@ -273,7 +273,7 @@ extern "C" int fr_moe_align(const void* topk_ids, int ids_dtype, int64_t n, int 
   FR_REQUIRE(E >= 1 && E <= kMaxE, FR_E_SHAPE, "fr_moe_align: E=%d outside [1, %d]", E, kMaxE);
   FR_REQUIRE(block >= 1 && block <= 4096, FR_E_SHAPE, "fr_moe_align: block=%d outside [1, 4096]", block);
   FR_REQUIRE(n + int64_t(E) * block < (int64_t(1) << 31), FR_E_SHAPE, "fr_moe_align: padded length overflows int32");
-  FR_REQUIRE(sorted_token_ids && expert_ids && num_tokens_post_pad, FR_E_NULL, "fr_moe_align: null output pointer");
+  FR_REQUIRE(expert_ids && num_tokens_post_pad && (sorted_token_ids || n + int64_t(E) * (block - 1) == 0), FR_E_NULL, "fr_moe_align: null output pointer");
   FR_REQUIRE(n == 0 || topk_ids, FR_E_NULL, "fr_moe_align: null topk_ids");
   FR_REQUIRE(ids_dtype == FR_I32 || ids_dtype == FR_I64, FR_E_DTYPE, "fr_moe_align: ids dtype %d not in {i32, i64}", ids_dtype);
   const int64_t need = fr_moe_align_workspace_bytes(n, E);

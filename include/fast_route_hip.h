@@ -86,7 +86,7 @@ int fr_moe_align(const void* topk_ids, int ids_dtype, int64_t n, int E, int bloc
  *   A [*, K] (row stride lda), B [E, N, K] dense, C [num_valid, N] dense.
  * Replaces: invoke_fused_moe_kernel / fused_moe_kernel,
  * fast_route/fast_route/ops/fused_moe.py:178-214 and :10-130.
- * Limits: K % 32 == 0, N % 4 == 0, block in {16, 32, 64, 128}; dtype in {FR_F16, FR_BF16}. */
+ * Limits: K % 64 == 0, N % 4 == 0, block in {16, 32, 64, 128, 256}; dtype in {FR_F16, FR_BF16}. */
 int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, void* C,
                         const float* topk_weights, const int32_t* sorted_token_ids,
                         const int32_t* expert_ids, const int32_t* num_tokens_post_pad,
