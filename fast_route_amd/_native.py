@@ -35,6 +35,14 @@ SIGNATURES = {
                                     c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "fr_fused_experts": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                  c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_void_p]),
+    "fr_quant_e4m3_rows": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),
+    "fr_moe_gateup_silu_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                                       c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "fr_moe_down_combine_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p,
+                                        c_void_p, c_void_p]),
+    "fr_fused_moe_fp8": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64,
+                                 c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_void_p]),
     "fr_fused_moe": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int,
                              c_int, c_int, c_void_p, c_void_p, c_int64, c_void_p]),
 }

@@ -13,6 +13,10 @@ char* error_buffer();
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
 
+// per-row e4m3 quantisation; rows_dev (optional, device) bounds the rows actually touched
+int quant_rows(const void* x, int dtype, int64_t rows, const int32_t* rows_dev, int64_t K, int64_t ldx, void* q_out,
+               float* scale_out, hipStream_t st);
+
 #define FR_REQUIRE(cond, code, ...) \
   do {                              \
     if (!(cond)) return ::fr::fail((code), __VA_ARGS__); \
@@ -37,6 +41,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
+struct __attribute__((aligned(16))) u32x4_t { unsigned x, y, z, w; };
 
 constexpr int kWave = 64;
 

@@ -18,10 +18,15 @@ struct Carve {
   int64_t align_ws_bytes;
   void* act;
   float* partial;
+  void* xq;          // fp8 layer only
+  float* x_scale;
+  void* actq;
+  float* act_scale;
   int64_t total;
 };
 
-int elem_size(int dtype) { return (dtype == FR_F16 || dtype == FR_BF16) ? 2 : (dtype == FR_F32 ? 4 : 1); }
+// the activated intermediate is stored in half precision also on the fp8 path
+int act_elem_size(int) { return 2; }
 
 Carve carve(void* base, int64_t M, int64_t H, int64_t F, int E, int topk, int dtype, const fr_moe_plan& p) {
   Carve c;
@@ -36,14 +41,21 @@ Carve carve(void* base, int64_t M, int64_t H, int64_t F, int E, int topk, int dt
   c.npost = reinterpret_cast<int32_t*>(take(4));
   c.align_ws_bytes = fr_moe_align_workspace_bytes(n, E);
   c.align_ws = take(c.align_ws_bytes);
-  c.act = take(p.sorted_len * F * elem_size(dtype));
+  c.act = take(p.sorted_len * F * act_elem_size(dtype));
   c.partial = reinterpret_cast<float*>(take(static_cast<int64_t>(p.split_k) * n * H * 4));
+  c.xq = nullptr; c.x_scale = nullptr; c.actq = nullptr; c.act_scale = nullptr;
+  if (dtype == FR_FP8_E4M3) {
+    c.xq = take(M * H);
+    c.x_scale = reinterpret_cast<float*>(take(M * 4));
+    c.actq = take(p.sorted_len * F);
+    c.act_scale = reinterpret_cast<float*>(take(p.sorted_len * 4));
+  }
   c.total = off;
   return c;
 }
 
 int check_layer_shapes(const char* who, int64_t M, int64_t H, int64_t F, int E, int topk, int dtype) {
-  FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "%s: dtype %d not in {f16, bf16}", who, dtype);
+  FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16 || dtype == FR_FP8_E4M3, FR_E_DTYPE, "%s: dtype %d not in {f16, bf16, fp8_e4m3}", who, dtype);
   FR_REQUIRE(M >= 0 && H > 0 && F > 0, FR_E_SHAPE, "%s: M=%lld H=%lld F=%lld", who, (long long)M, (long long)H, (long long)F);
   FR_REQUIRE(E >= 1 && E <= 1024 && topk >= 1 && topk <= E, FR_E_SHAPE, "%s: E=%d topk=%d", who, E, topk);
   FR_REQUIRE(H % 128 == 0 && F % 128 == 0, FR_E_SHAPE, "%s: H=%lld and F=%lld must be multiples of 128", who, (long long)H, (long long)F);
@@ -114,4 +126,32 @@ extern "C" int fr_fused_moe(const void* x, const void* w1, const void* w2, const
   rc = fr_gating_topk(logits, logits_dtype, M, E, E, topk, renormalize, c.topk_w, c.topk_ids, stream);
   if (rc != FR_OK) return rc;
   return fr_fused_experts(x, w1, w2, c.topk_w, c.topk_ids, M, H, F, E, topk, dtype, out, workspace, workspace_bytes, stream);
+}
+
+extern "C" int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, const float* w1_scale, const void* w2q,
+                                const float* w2_scale, const void* logits, int logits_dtype, int64_t M, int64_t H,
+                                int64_t F, int E, int topk, int renormalize, void* out, void* workspace,
+                                int64_t workspace_bytes, void* stream) {
+  fr_moe_plan p;
+  int rc = fr_moe_get_plan(M, H, F, E, topk, FR_FP8_E4M3, &p);
+  if (rc != FR_OK) return rc;
+  if (M == 0) return FR_OK;
+  FR_REQUIRE(x_dtype == FR_BF16, FR_E_DTYPE, "fr_fused_moe_fp8: activations must be bf16 (dtype %d)", x_dtype);
+  FR_REQUIRE(x && w1q && w1_scale && w2q && w2_scale && logits && out, FR_E_NULL, "fr_fused_moe_fp8: null pointer");
+  FR_REQUIRE(workspace && workspace_bytes >= p.workspace_bytes, FR_E_WORKSPACE, "fr_fused_moe_fp8: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)p.workspace_bytes);
+  FR_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FR_E_ALIGN, "fr_fused_moe_fp8: workspace must be 256-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  Carve c = carve(workspace, M, H, F, E, topk, FR_FP8_E4M3, p);
+  rc = fr_gating_topk(logits, logits_dtype, M, E, E, topk, renormalize, c.topk_w, c.topk_ids, stream);
+  if (rc != FR_OK) return rc;
+  rc = fr_moe_align(c.topk_ids, FR_I32, M * topk, E, p.block, c.sorted, c.expert_ids, c.npost, c.align_ws, c.align_ws_bytes, stream);
+  if (rc != FR_OK) return rc;
+  rc = quant_rows(x, x_dtype, M, nullptr, H, H, c.xq, c.x_scale, st);
+  if (rc != FR_OK) return rc;
+  rc = fr_moe_gateup_silu_fp8(c.xq, c.x_scale, w1q, w1_scale, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, c.act, stream);
+  if (rc != FR_OK) return rc;
+  rc = quant_rows(c.act, FR_BF16, p.sorted_len, c.npost, F, F, c.actq, c.act_scale, st);
+  if (rc != FR_OK) return rc;
+  return fr_moe_down_combine_fp8(c.actq, c.act_scale, w2q, w2_scale, c.topk_w, c.sorted, c.expert_ids, c.npost, M, H, F, E,
+                                 topk, p.block, p.split_k, x_dtype, c.partial, out, stream);
 }

@@ -2,18 +2,17 @@
 //
 // One workgroup computes a tile of BT sorted slots (one routing block, hence
 // one expert) by BF output features.  Both operands are K-contiguous in HBM
-// (tokens [*, K], weights [E, N, K]); tiles of BK are staged through LDS in
-// 16-byte chunks under an XOR swizzle and fed to v_mfma with the WEIGHT rows as
-// the MFMA "A" operand and the TOKEN rows as "B", so a lane's accumulator
-// registers hold 4 consecutive output features of one token and the epilogue
-// stores 8/16-byte vectors.  Three epilogues:
+// (tokens [*, K], weights [E, N, K]); K tiles of BKB bytes per row are staged
+// through LDS in 16-byte chunks under an XOR swizzle and fed to v_mfma with the
+// WEIGHT rows as the MFMA "A" operand and the TOKEN rows as "B", so a lane's
+// accumulator registers hold 4 consecutive output features of one token and the
+// epilogue stores 8/16-byte vectors.  Element types: bf16, fp16
+// (v_mfma_f32_{32x32x16,16x16x32}) and OCP fp8 e4m3 (v_mfma_f32_{32x32x64,16x16x128}_f8f6f4,
+// per-row fp32 scales of both operands applied in the epilogue).  Epilogues:
 //   EPI_PLAIN  C[pair] = acc (* routed weight), scattered by sorted id
 //   EPI_SILU   W tile = BF/2 gate rows + the matching BF/2 up rows; writes
 //              silu(gate)*up at the slot's own row of act[sorted_len, F]
 //   EPI_DOWN   partial[split][pair] = acc * routed weight in fp32 (split-K slices)
-// Workgroup ids are first regrouped so that each XCD (ids congruent mod 8) gets
-// a contiguous range of tiles, then walked in groups of GROUP_T token blocks x
-// all feature tiles so co-resident workgroups share weight tiles in their L2.
 #pragma once
 #include "fr_common.h"
 
@@ -27,7 +26,7 @@ struct GemmArgs {
   const void* X;        // token rows [*, K]
   int64_t ldx;          // row stride of X in elements
   const void* W;        // [E, w_rows, K]
-  int64_t w_expert_stride;
+  int64_t w_expert_stride;  // elements between experts
   int64_t ldw;          // row stride of W in elements
   void* out;
   int64_t ldo;          // row stride of out in elements
@@ -36,6 +35,9 @@ struct GemmArgs {
   const int32_t* expert_ids;
   const int32_t* npost;
   const float* topk_w;  // flat [num_valid] or nullptr
+  const float* x_scale; // fp8 only: one scale per X row (indexed like the X rows)
+  const float* w_scale; // fp8 only: [E, w_rows]
+  int w_rows;           // rows of W per expert (scale indexing)
   int num_valid;        // n = M*topk
   int top_k;            // X row = sorted id / top_k; 0 => X row = slot index
   int N;                // output features (EPI_SILU: F, W has 2F rows)
@@ -48,57 +50,81 @@ struct GemmArgs {
 };
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+struct fp8_t { unsigned char bits; };  // OCP e4m3fn storage
 
-template <typename T> struct Mfma;
-template <> struct Mfma<bf16_t> {
-  typedef bf16x8 vec8;
-  typedef bf16x4 vec4;
-  static __device__ __forceinline__ f32x16 m32(vec8 a, vec8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+// Element traits: FC = 16-byte chunks one lane feeds to one MFMA, out_t = type the
+// half-precision epilogues store.
+template <typename T> struct Elem;
+template <> struct Elem<bf16_t> {
+  typedef bf16_t out_t;
+  typedef bf16x4 out4;
+  static constexpr int FC = 1;
+  static constexpr bool SCALED = false;
+  static __device__ __forceinline__ f32x16 m32(const u32x4* a, const u32x4* b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]), c, 0, 0, 0);
   }
-  static __device__ __forceinline__ f32x4 m16(vec8 a, vec8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  static __device__ __forceinline__ f32x4 m16(const u32x4* a, const u32x4* b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]), c, 0, 0, 0);
   }
 };
-template <> struct Mfma<f16_t> {
-  typedef f16x8 vec8;
-  typedef f16x4 vec4;
-  static __device__ __forceinline__ f32x16 m32(vec8 a, vec8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+template <> struct Elem<f16_t> {
+  typedef f16_t out_t;
+  typedef f16x4 out4;
+  static constexpr int FC = 1;
+  static constexpr bool SCALED = false;
+  static __device__ __forceinline__ f32x16 m32(const u32x4* a, const u32x4* b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c, 0, 0, 0);
   }
-  static __device__ __forceinline__ f32x4 m16(vec8 a, vec8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  static __device__ __forceinline__ f32x4 m16(const u32x4* a, const u32x4* b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c, 0, 0, 0);
+  }
+};
+template <> struct Elem<fp8_t> {
+  typedef bf16_t out_t;
+  typedef bf16x4 out4;
+  static constexpr int FC = 2;
+  static constexpr bool SCALED = true;
+  static __device__ __forceinline__ i32x8 join(const u32x4* p) {
+    return __builtin_bit_cast(i32x8, __builtin_shufflevector(p[0], p[1], 0, 1, 2, 3, 4, 5, 6, 7));
+  }
+  // format selectors 0 = e4m3 for both operands; scale operands 0 = no block scaling
+  static __device__ __forceinline__ f32x16 m32(const u32x4* a, const u32x4* b, f32x16 c) {
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(join(a), join(b), c, 0, 0, 0, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 m16(const u32x4* a, const u32x4* b, f32x4 c) {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(join(a), join(b), c, 0, 0, 0, 0, 0, 0);
   }
 };
 
 __device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); }
 
-// Tile configuration.  TILE = 32 uses v_mfma_f32_32x32x16, TILE = 16 v_mfma_f32_16x16x32.
-// WT x WF wavefronts split the BT x BF tile; MINB = workgroups per CU the register
-// allocation should allow.  STAGES == 0: tiles go HBM -> registers -> LDS with two
-// LDS buffers (one tile in flight).  STAGES >= 2: tiles go HBM -> LDS directly
-// (global_load_lds_dwordx4) through a ring of STAGES buffers that is refilled as soon
-// as a tile's last fragments are in registers, so STAGES tiles are in flight or landed.
-template <int BT_, int BF_, int BK_, int WT_, int WF_, int TILE_, int MINB_ = 1, int STAGES_ = 0>
+// Tile configuration.  BKB = bytes of K per row per tile (64 bf16 or 128 fp8 = 128 B,
+// the L2 line: shorter row segments halve the L2->LDS rate).  TILE = 32 uses the
+// 32x32 MFMA shapes, TILE = 16 the 16x16 ones.  WT x WF wavefronts split the BT x BF
+// tile; MINB = workgroups per CU the register allocation should allow.
+// STAGES == 0: tiles go HBM -> registers -> LDS with two LDS buffers (one tile in
+// flight).  STAGES >= 2: tiles go HBM -> LDS directly (global_load_lds_dwordx4)
+// through a ring of STAGES buffers that is refilled as soon as a tile's last
+// fragments are in registers, so STAGES tiles are in flight or landed.
+template <int BT_, int BF_, int BKB_, int WT_, int WF_, int TILE_, int MINB_ = 1, int STAGES_ = 0>
 struct Cfg {
-  static constexpr int BT = BT_, BF = BF_, BK = BK_, WT = WT_, WF = WF_, TILE = TILE_, MINB = MINB_;
+  static constexpr int BT = BT_, BF = BF_, BKB = BKB_, WT = WT_, WF = WF_, TILE = TILE_, MINB = MINB_;
   static constexpr int STAGES = STAGES_;
   static constexpr int NBUF = STAGES_ == 0 ? 2 : STAGES_;
   static constexpr int NT = WT * WF * kWave;       // threads
+  static constexpr int NW = NT / kWave;
   static constexpr int TT = BT / WT, TF = BF / WF; // per-wave tile
   static constexpr int IT = TT / TILE, JF = TF / TILE;
-  static constexpr int CPR = BK / 8;               // 16-byte chunks per row
-  static constexpr int KSTEP = (TILE == 32) ? 16 : 32;
+  static constexpr int CPR = BKB / 16;             // 16-byte chunks per row
   static constexpr int KGROUPS = 64 / TILE;        // lane groups along K in one MFMA
   static constexpr int XCH = BT * CPR, WCH = BF * CPR;
   static constexpr int XL = (XCH + NT - 1) / NT, WL = (WCH + NT - 1) / NT;
-  static constexpr int LDS_BYTES = NBUF * (BT + BF) * BK * 2;
-  static constexpr int NW = NT / kWave;
   static constexpr int XI = XCH / (kWave * NW), WI = WCH / (kWave * NW);  // direct-to-LDS loads per wave per tile
-  static_assert(STAGES_ == 0 || (STAGES_ >= 2 && XCH % (kWave * NW) == 0 && WCH % (kWave * NW) == 0), "direct-to-LDS tiles must split evenly over the wavefronts");
+  static constexpr int LDS_BYTES = NBUF * (BT + BF) * BKB;
   static_assert(TT % TILE == 0 && TF % TILE == 0, "wave tile must be a multiple of the MFMA tile");
   static_assert(NT % CPR == 0, "threads must cover whole rows");
-  static_assert(BK % KSTEP == 0, "BK must be a multiple of the MFMA K");
+  static_assert(STAGES_ == 0 || (STAGES_ >= 2 && XCH % (kWave * NW) == 0 && WCH % (kWave * NW) == 0),
+                "direct-to-LDS tiles must split evenly over the wavefronts");
 };
 
 // LDS is 64 banks x 4 B: a 16-lane phase of ds_read_b128 is conflict-free when its
@@ -113,22 +139,28 @@ __device__ __forceinline__ int swizzle(int row, int chunk) {
 
 template <typename T, typename C, int EPI>
 __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs a) {
-  typedef typename Mfma<T>::vec8 vec8;
-  typedef typename Mfma<T>::vec4 vec4;
+  typedef Elem<T> E;
+  typedef typename E::out_t out_t;
+  typedef typename E::out4 out4;
   typedef typename std::conditional<C::TILE == 32, f32x16, f32x4>::type acc_t;
-  constexpr int BT = C::BT, BF = C::BF, BK = C::BK, CPR = C::CPR, NT = C::NT;
+  constexpr int BT = C::BT, BF = C::BF, CPR = C::CPR, NT = C::NT, FC = E::FC;
+  constexpr int EPC = 16 / static_cast<int>(sizeof(T));     // elements per 16-byte chunk
+  constexpr int BK = C::BKB / static_cast<int>(sizeof(T));  // elements of K per tile
+  constexpr int KS = CPR / (C::KGROUPS * FC);               // MFMA K-steps per tile
   constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
+  static_assert(CPR % (C::KGROUPS * FC) == 0 && KS >= 1, "tile K must be a multiple of the MFMA K");
   static_assert(EPI != EPI_SILU || C::JF % 2 == 0, "gate and up tiles must pair up inside a wave");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   u32x4* lds = reinterpret_cast<u32x4*>(lds_raw);
-  // buffer b: X tile at b*BUF, W tile right after it
-  constexpr int BUF = C::XCH + C::WCH;
+  constexpr int BUF = C::XCH + C::WCH;  // buffer b: X tile at b*BUF, W tile right after it
 
   // ---- tile coordinates ---------------------------------------------------
   // The grid is sized for the worst-case padded length; only the first
   // (npost/BT)*num_f_tiles workgroups have a tile.  Tiles are dealt to the 8 XCDs
-  // (workgroup id mod 8) in contiguous, equally sized ranges of the REAL tile count.
+  // (workgroup id mod 8) in contiguous, equally sized ranges of the REAL tile
+  // count, then walked in groups of group_t token blocks x all feature tiles so
+  // co-resident workgroups share weight tiles in their XCD's L2.
   const int npost = a.npost[0];
   const int nt = min(npost / BT, a.num_t_blocks);
   const int total = nt * a.num_f_tiles;
@@ -151,15 +183,10 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wt = wave / C::WF, wf = wave % C::WF;
 
-  // ---- global source pointers for this thread's chunks ----------------------
   const T* X = static_cast<const T*>(a.X);
   const T* W = static_cast<const T*>(a.W) + static_cast<int64_t>(expert) * a.w_expert_stride;
   const int k0 = split * a.k_per_split;
   const int k_tiles = min(a.k_per_split, a.K - k0) / BK;
-  const int chunk = tid % CPR;
-  const int row0 = tid / CPR;
-  constexpr int ROWS_PER_PASS = NT / CPR;
-  constexpr bool X_FULL = (C::XCH % NT == 0), W_FULL = (C::WCH % NT == 0);
 
   // X row of a tile row (gathered through the routing arrays) and W row of a tile row
   auto x_src_row = [&](int rr) -> int64_t {
@@ -181,9 +208,9 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
 
   // ---- per-lane fragment rows ---------------------------------------------
   const int frow = lane % C::TILE;  // row inside an MFMA tile
-  const int kgrp = lane / C::TILE;  // which 8-element K group of the MFMA this lane feeds
-  int xoff[C::IT], woff[C::JF];     // chunk offset of the lane's row, swizzle key folded in below
-  int xkey[C::IT], wkey[C::JF];
+  const int kgrp = lane / C::TILE;  // which K group of the MFMA this lane feeds
+  int xoff[C::IT], woff[C::JF];     // chunk offset of the lane's row
+  int xkey[C::IT], wkey[C::JF];     // swizzle key of that row
 #pragma unroll
   for (int i = 0; i < C::IT; ++i) {
     const int r = wt * C::TT + i * C::TILE + frow;
@@ -212,51 +239,53 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
 #pragma unroll
       for (int r = 0; r < ACC_N; ++r) acc[j][i][r] = 0.f;
 
-#define FR_COMPUTE_TILE(buf)                                                          \
-  {                                                                                   \
-    const u32x4* tile = lds + (buf) * BUF;                                            \
-    _Pragma("unroll") for (int ks = 0; ks < BK / C::KSTEP; ++ks) {                    \
-      const int kc = ks * C::KGROUPS + kgrp;                                          \
-      vec8 xf[C::IT], wfr[C::JF];                                                     \
-      _Pragma("unroll") for (int i = 0; i < C::IT; ++i) {                             \
-        const u32x4 v = tile[xoff[i] + (kc ^ xkey[i])];                               \
-        xf[i] = __builtin_bit_cast(vec8, v);                                          \
-      }                                                                               \
-      _Pragma("unroll") for (int j = 0; j < C::JF; ++j) {                             \
-        const u32x4 v = tile[woff[j] + (kc ^ wkey[j])];                               \
-        wfr[j] = __builtin_bit_cast(vec8, v);                                         \
-      }                                                                               \
-      _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                               \
-        _Pragma("unroll") for (int i = 0; i < C::IT; ++i) {                           \
-          if constexpr (C::TILE == 32) acc[j][i] = Mfma<T>::m32(wfr[j], xf[i], acc[j][i]); \
-          else acc[j][i] = Mfma<T>::m16(wfr[j], xf[i], acc[j][i]);                    \
-        }                                                                             \
-    }                                                                                 \
+  // fragments, double-buffered in registers: [buffer][tile][chunk]
+  u32x4 xf[2][C::IT][FC], wfr[2][C::JF][FC];
+#define FR_READ_FRAGS(stage_, ks_, fb_)                                                 \
+  {                                                                                     \
+    const u32x4* tile = lds + (stage_) * BUF;                                           \
+    _Pragma("unroll") for (int c = 0; c < FC; ++c) {                                    \
+      const int kc = ((ks_) * C::KGROUPS + kgrp) * FC + c;                              \
+      _Pragma("unroll") for (int i = 0; i < C::IT; ++i)                                 \
+        xf[fb_][i][c] = tile[xoff[i] + (kc ^ xkey[i])];                                 \
+      _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                                 \
+        wfr[fb_][j][c] = tile[woff[j] + (kc ^ wkey[j])];                                \
+    }                                                                                   \
   }
-
+#define FR_MMA(fb_, j0_, j1_)                                                           \
+  {                                                                                     \
+    _Pragma("unroll") for (int j = (j0_); j < (j1_); ++j)                               \
+      _Pragma("unroll") for (int i = 0; i < C::IT; ++i) {                               \
+        if constexpr (C::TILE == 32) acc[j][i] = E::m32(wfr[fb_][j], xf[fb_][i], acc[j][i]); \
+        else acc[j][i] = E::m16(wfr[fb_][j], xf[fb_][i], acc[j][i]);                    \
+      }                                                                                 \
+  }
 
   if constexpr (C::STAGES == 0) {
-  const T* xsrc[C::XL];
-  int xdst[C::XL];
+    // ---- register-staged double buffering ------------------------------------
+    const int chunk = tid % CPR;
+    const int row0 = tid / CPR;
+    constexpr int ROWS_PER_PASS = NT / CPR;
+    constexpr bool X_FULL = (C::XCH % NT == 0), W_FULL = (C::WCH % NT == 0);
+    const T* xsrc[C::XL];
+    int xdst[C::XL];
 #pragma unroll
-  for (int i = 0; i < C::XL; ++i) {
-    const int r = row0 + i * ROWS_PER_PASS;
-    const int rr = r < BT ? r : BT - 1;
-    xsrc[i] = X + x_src_row(rr) * a.ldx + k0 + chunk * 8;
-    xdst[i] = rr * CPR + swizzle<CPR>(rr, chunk);
-  }
-  const T* wsrc[C::WL];
-  int wdst[C::WL];
+    for (int i = 0; i < C::XL; ++i) {
+      const int r = row0 + i * ROWS_PER_PASS;
+      const int rr = r < BT ? r : BT - 1;
+      xsrc[i] = X + x_src_row(rr) * a.ldx + k0 + chunk * EPC;
+      xdst[i] = rr * CPR + swizzle<CPR>(rr, chunk);
+    }
+    const T* wsrc[C::WL];
+    int wdst[C::WL];
 #pragma unroll
-  for (int i = 0; i < C::WL; ++i) {
-    const int r = row0 + i * ROWS_PER_PASS;
-    const int rr = r < BF ? r : BF - 1;
-    wsrc[i] = W + static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + chunk * 8;
-    wdst[i] = C::XCH + rr * CPR + swizzle<CPR>(rr, chunk);
-  }
-
-  u32x4 xreg[C::XL], wreg[C::WL];
-
+    for (int i = 0; i < C::WL; ++i) {
+      const int r = row0 + i * ROWS_PER_PASS;
+      const int rr = r < BF ? r : BF - 1;
+      wsrc[i] = W + static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + chunk * EPC;
+      wdst[i] = C::XCH + rr * CPR + swizzle<CPR>(rr, chunk);
+    }
+    u32x4 xreg[C::XL], wreg[C::WL];
 #define FR_LOAD_TILE(kt)                                                              \
   {                                                                                   \
     _Pragma("unroll") for (int i = 0; i < C::XL; ++i)                                 \
@@ -273,23 +302,29 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     _Pragma("unroll") for (int i = 0; i < C::WL; ++i)                                 \
       if (W_FULL || row0 + i * ROWS_PER_PASS < BF) lds[(buf) * BUF + wdst[i]] = wreg[i]; \
   }
-  // ---- main loop: register-staged double buffering, last tile peeled ---------
-  FR_LOAD_TILE(0);
-  FR_STORE_TILE(0);
-  __syncthreads();
-  for (int kt = 0; kt < k_tiles - 1; ++kt) {
-    const int buf = kt & 1;
-    FR_LOAD_TILE(kt + 1);
-    __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the MFMA block
-    FR_COMPUTE_TILE(buf);
-    __builtin_amdgcn_sched_barrier(0);
-    FR_STORE_TILE(buf ^ 1);
-    __syncthreads();
+#define FR_COMPUTE_TILE(buf)                                                          \
+  {                                                                                   \
+    _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                               \
+      FR_READ_FRAGS(buf, ks, 0);                                                      \
+      FR_MMA(0, 0, C::JF);                                                            \
+    }                                                                                 \
   }
-  FR_COMPUTE_TILE((k_tiles - 1) & 1);
+    FR_LOAD_TILE(0);
+    FR_STORE_TILE(0);
+    __syncthreads();
+    for (int kt = 0; kt < k_tiles - 1; ++kt) {
+      const int buf = kt & 1;
+      FR_LOAD_TILE(kt + 1);
+      __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the MFMA block
+      FR_COMPUTE_TILE(buf);
+      __builtin_amdgcn_sched_barrier(0);
+      FR_STORE_TILE(buf ^ 1);
+      __syncthreads();
+    }
+    FR_COMPUTE_TILE((k_tiles - 1) & 1);
 #undef FR_LOAD_TILE
 #undef FR_STORE_TILE
-
+#undef FR_COMPUTE_TILE
   } else {
     // ---- direct-to-LDS ring --------------------------------------------------
     // A wavefront-wide global_load_lds_dwordx4 fills 64 consecutive 16-byte LDS
@@ -297,12 +332,9 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     // lane fetches the logical chunk that the swizzle maps to its slot.
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI;
-#ifdef FR_TUNE_XI
-    constexpr int LPT = FR_TUNE_XI + FR_TUNE_WI;
-#else
-    constexpr int LPT = XI + WI;
-#endif
+    constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, LPT = XI + WI;
+    static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
+    static_assert(S <= 5 && (S - 1) * LPT <= 63, "vmcnt budget");
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const T* xsrc[XI];
     const T* wsrc[WI];
@@ -310,25 +342,21 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     for (int i = 0; i < XI; ++i) {
       const int slot = (i * NW + wave_u) * kWave + lane;
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
-      xsrc[i] = X + x_src_row(rr) * a.ldx + k0 + c * 8;
+      xsrc[i] = X + x_src_row(rr) * a.ldx + k0 + c * EPC;
     }
 #pragma unroll
     for (int i = 0; i < WI; ++i) {
       const int slot = (i * NW + wave_u) * kWave + lane;
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
-      wsrc[i] = W + static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * 8;
+      wsrc[i] = W + static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * EPC;
     }
-#ifndef FR_TUNE_XI
-#define FR_TUNE_XI XI
-#define FR_TUNE_WI WI
-#endif
 #define FR_ISSUE_TILE(kt, stage)                                                                    \
   {                                                                                                 \
     unsigned char* sbase = lds_raw + (stage) * (BUF * 16);                                          \
-    _Pragma("unroll") for (int i = 0; i < FR_TUNE_XI; ++i)                                          \
+    _Pragma("unroll") for (int i = 0; i < XI; ++i)                                                  \
       __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[i] + (kt) * BK),                               \
                                        (lptr_t)(sbase + (i * NW + wave_u) * (kWave * 16)), 16, 0, 0); \
-    _Pragma("unroll") for (int i = 0; i < FR_TUNE_WI; ++i)                                          \
+    _Pragma("unroll") for (int i = 0; i < WI; ++i)                                                  \
       __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + (kt) * BK),                               \
                                        (lptr_t)(sbase + C::XCH * 16 + (i * NW + wave_u) * (kWave * 16)), 16, 0, 0); \
   }
@@ -340,43 +368,6 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
       else if (tiles_after == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
       else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     };
-    static_assert(S <= 5 && (S - 1) * LPT <= 63, "vmcnt budget");
-    // Software pipeline: fragments are double-buffered in registers; while the
-    // MFMAs of K-step ks run, the ds_reads of K-step ks+1 are in flight.  The
-    // barrier that publishes tile kt+1 sits before the LAST K-step of tile kt,
-    // whose fragments are already in registers, so no wavefront waits on LDS
-    // latency right after a barrier.
-    constexpr int KS = BK / C::KSTEP;
-    static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
-    vec8 xf[2][C::IT], wfr[2][C::JF];
-#ifdef FR_TUNE_NO_READ
-#define FR_READ_FRAGS(stage_, ks_, fb_) { if ((ks_) == 100) { xf[fb_][0] = __builtin_bit_cast(vec8, lds[stage_]); } }
-#else
-#define FR_READ_FRAGS(stage_, ks_, fb_)                                                 \
-  {                                                                                     \
-    const u32x4* tile = lds + (stage_) * BUF;                                           \
-    const int kc = (ks_) * C::KGROUPS + kgrp;                                           \
-    _Pragma("unroll") for (int i = 0; i < C::IT; ++i)                                   \
-      xf[fb_][i] = __builtin_bit_cast(vec8, tile[xoff[i] + (kc ^ xkey[i])]);            \
-    _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                                   \
-      wfr[fb_][j] = __builtin_bit_cast(vec8, tile[woff[j] + (kc ^ wkey[j])]);           \
-  }
-#endif
-#ifdef FR_TUNE_NO_MMA  /* bottleneck bisection builds only: one MFMA per call keeps the fragments live */
-#define FR_MMA(fb_, j0_, j1_)                                                           \
-  {                                                                                     \
-    if ((j0_) == 0) { _Pragma("unroll") for (int i = 0; i < C::IT; ++i) _Pragma("unroll") for (int j = 0; j < C::JF; ++j) { acc[j][i][0] += __builtin_bit_cast(f32x4, xf[fb_][i])[0] + __builtin_bit_cast(f32x4, wfr[fb_][j])[0]; } } \
-  }
-#else
-#define FR_MMA(fb_, j0_, j1_)                                                           \
-  {                                                                                     \
-    _Pragma("unroll") for (int j = (j0_); j < (j1_); ++j)                               \
-      _Pragma("unroll") for (int i = 0; i < C::IT; ++i) {                               \
-        if constexpr (C::TILE == 32) acc[j][i] = Mfma<T>::m32(wfr[fb_][j], xf[fb_][i], acc[j][i]); \
-        else acc[j][i] = Mfma<T>::m16(wfr[fb_][j], xf[fb_][i], acc[j][i]);              \
-      }                                                                                 \
-  }
-#endif
     // One K-step: first MFMAs of the step, then the ds_reads of the NEXT step (other
     // fragment buffer), then the remaining MFMAs, which cover the LDS latency.
     constexpr int JSPLIT = (C::JF + 1) / 2;
@@ -390,6 +381,9 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     FR_MMA(fb_, JSPLIT, C::JF);                  \
     __builtin_amdgcn_sched_barrier(0);           \
   }
+    // Software pipeline: the barrier that publishes tile kt+1 sits before the LAST
+    // K-step of tile kt, whose fragments are already in registers; the slot of tile
+    // kt is refilled right after that barrier.
 #pragma unroll
     for (int t = 0; t < S; ++t)
       if (t < k_tiles) FR_ISSUE_TILE(t, t);
@@ -440,63 +434,81 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
         FR_KSTEP(ks & 1, {});
       }
     }
-#undef FR_READ_FRAGS
-#undef FR_MMA
 #undef FR_KSTEP
 #undef FR_ISSUE_TILE
   }
-#undef FR_COMPUTE_TILE
+#undef FR_READ_FRAGS
+#undef FR_MMA
 
   // ---- epilogue -------------------------------------------------------------
   // lane holds token column (lane % TILE) of each token tile and, per accumulator
   // group g (TILE==32: 4 groups of 4 regs; TILE==16: one), 4 consecutive features
   // starting at g*8 + kgrp*4 (TILE==32) or kgrp*4 (TILE==16) inside the MFMA tile.
   constexpr int GROUPS = ACC_N / 4;
+  const float* wsc = nullptr;
+  if constexpr (E::SCALED) wsc = a.w_scale + static_cast<int64_t>(expert) * a.w_rows;
 #pragma unroll
   for (int i = 0; i < C::IT; ++i) {
     const int slot = pid_t * BT + wt * C::TT + i * C::TILE + frow;
+    int sid = 0;
+    if constexpr (EPI != EPI_SILU || E::SCALED) sid = a.sorted[slot];
+    float xs = 1.f;
+    if constexpr (E::SCALED) {
+      if (a.top_k > 0) xs = sid < a.num_valid ? a.x_scale[sid / a.top_k] : 1.f;
+      else xs = a.x_scale[slot];
+    }
     if constexpr (EPI == EPI_SILU) {
       constexpr int HJ = C::JF / 2;
-      T* orow = static_cast<T*>(a.out) + static_cast<int64_t>(slot) * a.ldo;
+      out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(slot) * a.ldo;
 #pragma unroll
       for (int j = 0; j < HJ; ++j)
 #pragma unroll
         for (int g = 0; g < GROUPS; ++g) {
           const int f = pid_f * (BF / 2) + wf * (C::TF / 2) + j * C::TILE + g * 8 + kgrp * 4;
-          vec4 o;
+          out4 o;
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            o[r] = static_cast<T>(silu(acc[j][i][g * 4 + r]) * acc[j + HJ][i][g * 4 + r]);
-          if (f + 3 < a.N) *reinterpret_cast<vec4*>(orow + f) = o;
+          for (int r = 0; r < 4; ++r) {
+            float gv = acc[j][i][g * 4 + r], uv = acc[j + HJ][i][g * 4 + r];
+            if constexpr (E::SCALED) {
+              const int fc = f + r < a.N ? f + r : a.N - 1;
+              gv *= xs * wsc[fc];
+              uv *= xs * wsc[a.N + fc];
+            }
+            o[r] = static_cast<out_t>(silu(gv) * uv);
+          }
+          if (f + 3 < a.N) *reinterpret_cast<out4*>(orow + f) = o;
           else
             for (int r = 0; r < 4; ++r)
               if (f + r < a.N) orow[f + r] = o[r];
         }
     } else {
-      const int sid = a.sorted[slot];
       if (sid < a.num_valid) {
-        const float rw = a.mul_weight ? a.topk_w[sid] : 1.f;
+        const float rw = (a.mul_weight ? a.topk_w[sid] : 1.f) * xs;
 #pragma unroll
         for (int j = 0; j < C::JF; ++j)
 #pragma unroll
           for (int g = 0; g < GROUPS; ++g) {
             const int f = pid_f * BF + wf * C::TF + j * C::TILE + g * 8 + kgrp * 4;
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              v[r] = acc[j][i][g * 4 + r] * rw;
+              if constexpr (E::SCALED) v[r] *= wsc[f + r < a.N ? f + r : a.N - 1];
+            }
             if constexpr (EPI == EPI_DOWN) {
               float* orow = static_cast<float*>(a.out) + static_cast<int64_t>(split) * a.split_stride +
                             static_cast<int64_t>(sid) * a.ldo;
-              f32x4 o;
-#pragma unroll
-              for (int r = 0; r < 4; ++r) o[r] = acc[j][i][g * 4 + r] * rw;
+              const f32x4 o = {v[0], v[1], v[2], v[3]};
               if (f + 3 < a.N) *reinterpret_cast<f32x4*>(orow + f) = o;
               else
                 for (int r = 0; r < 4; ++r)
-                  if (f + r < a.N) orow[f + r] = o[r];
+                  if (f + r < a.N) orow[f + r] = v[r];
             } else {
-              T* orow = static_cast<T*>(a.out) + static_cast<int64_t>(sid) * a.ldo;
-              vec4 o;
+              out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(sid) * a.ldo;
+              out4 o;
 #pragma unroll
-              for (int r = 0; r < 4; ++r) o[r] = static_cast<T>(acc[j][i][g * 4 + r] * rw);
-              if (f + 3 < a.N) *reinterpret_cast<vec4*>(orow + f) = o;
+              for (int r = 0; r < 4; ++r) o[r] = static_cast<out_t>(v[r]);
+              if (f + 3 < a.N) *reinterpret_cast<out4*>(orow + f) = o;
               else
                 for (int r = 0; r < 4; ++r)
                   if (f + r < a.N) orow[f + r] = o[r];

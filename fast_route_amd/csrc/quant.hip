@@ -1,0 +1,103 @@
+// Per-row dynamic quantisation to OCP fp8 e4m3 on gfx950.
+//
+// One wavefront per row: pass 1 reduces max|x| across the row (16-byte loads,
+// cross-lane butterfly), scale = amax/448 (1 for an all-zero row); pass 2
+// re-reads the row (L2-resident) and converts x/scale with v_cvt_pk_fp8_f32
+// (round to nearest even), 16 codes per 16-byte store.
+#include "fr_common.h"
+
+namespace fr {
+namespace {
+
+constexpr int kQuantThreads = 256;
+constexpr int kQuantRowsPerBlock = kQuantThreads / kWave;
+
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16_t> { typedef bf16x8 type; };
+template <> struct Vec8<f16_t> { typedef f16x8 type; };
+
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, partner_f32<1>(v));
+  v = fmaxf(v, partner_f32<2>(v));
+  v = fmaxf(v, partner_f32<4>(v));
+  v = fmaxf(v, partner_f32<8>(v));
+  v = fmaxf(v, partner_f32<16>(v));
+  v = fmaxf(v, partner_f32<32>(v));
+  return v;
+}
+
+__device__ __forceinline__ unsigned pack4(float a, float b, float c, float d) {
+  int w = 0;
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  return static_cast<unsigned>(w);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kQuantThreads) void quant_rows_kernel(const T* __restrict__ x, int64_t rows,
+                                                                   const int32_t* __restrict__ rows_dev, int K,
+                                                                   int64_t ldx, unsigned char* __restrict__ q,
+                                                                   float* __restrict__ scale) {
+  typedef typename Vec8<T>::type vec8;
+  const int lane = threadIdx.x % kWave;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kQuantRowsPerBlock + threadIdx.x / kWave;
+  if (row >= rows || (rows_dev && row >= rows_dev[0])) return;
+  const T* xr = x + row * ldx;
+  float amax = 0.f;
+  for (int k = lane * 8; k < K; k += kWave * 8) {
+    const vec8 v = *reinterpret_cast<const vec8*>(xr + k);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(static_cast<float>(v[i])));
+  }
+  amax = wave_max(amax);
+  const float s = amax > 0.f ? amax / 448.f : 1.f;
+  if (lane == 0) scale[row] = s;
+  unsigned char* qr = q + row * static_cast<int64_t>(K);
+  for (int k = lane * 16; k < K; k += kWave * 16) {
+    const vec8 v0 = *reinterpret_cast<const vec8*>(xr + k);
+    const vec8 v1 = *reinterpret_cast<const vec8*>(xr + k + 8);
+    float f[16];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      f[i] = fminf(fmaxf(static_cast<float>(v0[i]) / s, -448.f), 448.f);
+      f[8 + i] = fminf(fmaxf(static_cast<float>(v1[i]) / s, -448.f), 448.f);
+    }
+    u32x4_t o;
+    o.x = pack4(f[0], f[1], f[2], f[3]);
+    o.y = pack4(f[4], f[5], f[6], f[7]);
+    o.z = pack4(f[8], f[9], f[10], f[11]);
+    o.w = pack4(f[12], f[13], f[14], f[15]);
+    *reinterpret_cast<u32x4_t*>(qr + k) = o;
+  }
+}
+
+}  // namespace
+}  // namespace fr
+
+namespace fr {
+// rows_dev (optional, device): only rows below *rows_dev are touched
+int quant_rows(const void* x, int dtype, int64_t rows, const int32_t* rows_dev, int64_t K, int64_t ldx, void* q_out,
+               float* scale_out, hipStream_t st) {
+  if (rows == 0) return FR_OK;
+  const unsigned grid = static_cast<unsigned>(ceil_div(rows, kQuantRowsPerBlock));
+  if (dtype == FR_BF16)
+    hipLaunchKernelGGL(quant_rows_kernel<bf16_t>, dim3(grid), dim3(kQuantThreads), 0, st, static_cast<const bf16_t*>(x), rows, rows_dev, (int)K, ldx, static_cast<unsigned char*>(q_out), scale_out);
+  else if (dtype == FR_F16)
+    hipLaunchKernelGGL(quant_rows_kernel<f16_t>, dim3(grid), dim3(kQuantThreads), 0, st, static_cast<const f16_t*>(x), rows, rows_dev, (int)K, ldx, static_cast<unsigned char*>(q_out), scale_out);
+  else
+    return fail(FR_E_DTYPE, "quantisation source dtype %d not in {f16, bf16}", dtype);
+  return check_launch("quant_rows_kernel");
+}
+}  // namespace fr
+
+extern "C" int fr_quant_e4m3_rows(const void* x, int dtype, int64_t rows, int64_t K, int64_t ldx, void* q_out,
+                                  float* scale_out, void* stream) {
+  using namespace fr;
+  FR_REQUIRE(rows >= 0, FR_E_SHAPE, "fr_quant_e4m3_rows: rows=%lld < 0", (long long)rows);
+  if (rows == 0) return FR_OK;
+  FR_REQUIRE(x && q_out && scale_out, FR_E_NULL, "fr_quant_e4m3_rows: null pointer");
+  FR_REQUIRE(K > 0 && K % 16 == 0 && K < (int64_t(1) << 30), FR_E_SHAPE, "fr_quant_e4m3_rows: K=%lld must be a positive multiple of 16", (long long)K);
+  FR_REQUIRE(ldx >= K && ldx % 8 == 0 && aligned16(x) && aligned16(q_out), FR_E_ALIGN, "fr_quant_e4m3_rows: 16-byte alignment, ldx %% 8 == 0, ldx >= K");
+  FR_REQUIRE(dtype == FR_BF16 || dtype == FR_F16, FR_E_DTYPE, "fr_quant_e4m3_rows: dtype %d not in {f16, bf16}", dtype);
+  return quant_rows(x, dtype, rows, nullptr, K, ldx, q_out, scale_out, static_cast<hipStream_t>(stream));
+}

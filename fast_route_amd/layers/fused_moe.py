@@ -19,9 +19,9 @@ def _check_layer(hidden_states, w1, w2):
     N.require_cuda(hidden_states, w1, w2)
 
 
-def plan(M: int, H: int, F: int, E: int, topk: int, dtype) -> N.FrMoePlan:
+def plan(M: int, H: int, F: int, E: int, topk: int, dtype, code: int | None = None) -> N.FrMoePlan:
     p = N.FrMoePlan()
-    N.check(N.lib().fr_moe_get_plan(M, H, F, E, topk, N.dtype_code(dtype), p))
+    N.check(N.lib().fr_moe_get_plan(M, H, F, E, topk, N.dtype_code(dtype) if code is None else code, p))
     return p
 
 

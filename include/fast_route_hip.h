@@ -142,6 +142,42 @@ int fr_fused_moe(const void* x, const void* w1, const void* w2, const void* logi
                  int renormalize, int dtype, void* out, void* workspace, int64_t workspace_bytes,
                  void* stream);
 
+/* ---- fp8 (OCP e4m3fn) path -------------------------------------------------
+ * No counterpart in the reference (its only fp8 mentions are commented autotune
+ * rows, fast_route/fast_route/ops/stable_route.py:20-28); defined by the fp8
+ * workload of this build: weights quantised per (expert, output channel),
+ * activations per token, fp32 scales, fp32 accumulation on the f8f6f4 MFMAs.
+ *
+ * Per-row dynamic quantisation: scale[r] = max|x[r,:]|/448 (1 for a zero row),
+ * q[r,:] = e4m3(x[r,:]/scale[r]) with round-to-nearest-even.  x is f16/bf16
+ * [rows, K] with row stride ldx; q is uint8 [rows, K] dense.  K % 16 == 0.
+ * Use it on w1 viewed as [E*2F, H] and w2 as [E*H, F] to prepare weights. */
+int fr_quant_e4m3_rows(const void* x, int dtype, int64_t rows, int64_t K, int64_t ldx, void* q_out,
+                       float* scale_out, void* stream);
+
+/* fp8 forms of fr_moe_gateup_silu / fr_moe_down_combine: operands are e4m3
+ * codes with one fp32 scale per row (x_scale[M], w1_scale[E, 2F], act_scale
+ * [sorted_len], w2_scale[E, H]); act is written / read in bf16 resp. e4m3;
+ * H and F must be multiples of 128. */
+int fr_moe_gateup_silu_fp8(const void* xq, const float* x_scale, const void* w1q, const float* w1_scale,
+                           const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                           const int32_t* num_tokens_post_pad, int64_t M, int64_t H, int64_t F, int E,
+                           int topk, int block, void* act_bf16, void* stream);
+int fr_moe_down_combine_fp8(const void* actq, const float* act_scale, const void* w2q, const float* w2_scale,
+                            const float* topk_weights, const int32_t* sorted_token_ids,
+                            const int32_t* expert_ids, const int32_t* num_tokens_post_pad, int64_t M,
+                            int64_t H, int64_t F, int E, int topk, int block, int split_k, int out_dtype,
+                            float* partial, void* out, void* stream);
+
+/* Whole fp8 layer from bf16 activations and router logits: gating, routing,
+ * per-token quantisation of x, fp8 gate/up GEMM + SiLU*mul (bf16 act), per-row
+ * quantisation of act, fp8 down GEMM + routed weight + combine.  Workspace size:
+ * fr_moe_get_plan(..., FR_FP8_E4M3, &plan).workspace_bytes. */
+int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, const float* w1_scale, const void* w2q,
+                     const float* w2_scale, const void* logits, int logits_dtype, int64_t M, int64_t H,
+                     int64_t F, int E, int topk, int renormalize, void* out, void* workspace,
+                     int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
