@@ -23,6 +23,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 SHAPES = {
     "mixtral": dict(H=4096, F=14336, E=8, topk=2, zipf=False, sweep=[1, 16, 64, 256, 1024, 4096, 16384]),
@@ -45,8 +46,9 @@ def layer_bytes(M, H, F, E, topk, active, bw=2, ba=2):
 class Layer:
     """Device buffers + staged calls through the C ABI for one (shape, M)."""
 
-    def __init__(self, torch, N, shape, M, w1, w2, seed):
+    def __init__(self, torch, N, shape, M, w1, w2, seed, fp8=None):
         self.torch, self.N, self.M = torch, N, M
+        self.fp8 = fp8  # (w1q, w1_scale, w2q, w2_scale) or None
         self.H, self.F, self.E, self.topk = shape["H"], shape["F"], shape["E"], shape["topk"]
         dev = "cuda"
         g = torch.Generator(device=dev).manual_seed(seed + M)
@@ -59,7 +61,7 @@ class Layer:
             self.logits = torch.randn(M, self.E, generator=g, device=dev)
         self.w1, self.w2 = w1, w2
         self.plan = N.FrMoePlan()
-        N.check(N.lib().fr_moe_get_plan(M, self.H, self.F, self.E, self.topk, N.FR_BF16, self.plan))
+        N.check(N.lib().fr_moe_get_plan(M, self.H, self.F, self.E, self.topk, N.FR_FP8_E4M3 if fp8 else N.FR_BF16, self.plan))
         p, n = self.plan, M * self.topk
         self.ws = torch.empty(max(p.workspace_bytes, 256), dtype=torch.uint8, device=dev)
         self.out = torch.empty(M, self.H, dtype=torch.bfloat16, device=dev)
@@ -73,10 +75,21 @@ class Layer:
         self.aws = torch.empty(max(self.aws_bytes, 256), dtype=torch.uint8, device=dev)
         self.act = torch.empty(p.sorted_len, self.F, dtype=torch.bfloat16, device=dev)
         self.partial = torch.empty(p.split_k * n * self.H, dtype=torch.float32, device=dev)
+        if fp8:
+            self.xq = torch.empty(M, self.H, dtype=torch.uint8, device=dev)
+            self.xs = torch.empty(M, dtype=torch.float32, device=dev)
+            self.actq = torch.empty(p.sorted_len, self.F, dtype=torch.uint8, device=dev)
+            self.acts = torch.ones(p.sorted_len, dtype=torch.float32, device=dev)
         self.stream = torch.cuda.current_stream().cuda_stream
 
     def fused(self):
         N = self.N
+        if self.fp8:
+            w1q, w1s, w2q, w2s = self.fp8
+            N.check(N.lib().fr_fused_moe_fp8(self.x.data_ptr(), N.FR_BF16, w1q.data_ptr(), w1s.data_ptr(), w2q.data_ptr(),
+                                             w2s.data_ptr(), self.logits.data_ptr(), N.FR_F32, self.M, self.H, self.F, self.E,
+                                             self.topk, 1, self.out.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream))
+            return
         N.check(N.lib().fr_fused_moe(self.x.data_ptr(), self.w1.data_ptr(), self.w2.data_ptr(), self.logits.data_ptr(),
                                      N.FR_F32, self.M, self.H, self.F, self.E, self.topk, 1, N.FR_BF16,
                                      self.out.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream))
@@ -91,6 +104,22 @@ class Layer:
         N.check(lib.fr_moe_align(self.ti.data_ptr(), N.FR_I32, self.M * self.topk, self.E, p.block, self.sorted.data_ptr(),
                                  self.eids.data_ptr(), self.npost.data_ptr(), self.aws.data_ptr(), self.aws_bytes, self.stream))
         rec(2)
+        if self.fp8:
+            w1q, w1s, w2q, w2s = self.fp8
+            N.check(lib.fr_quant_e4m3_rows(self.x.data_ptr(), N.FR_BF16, self.M, self.H, self.H, self.xq.data_ptr(),
+                                           self.xs.data_ptr(), self.stream))
+            N.check(lib.fr_moe_gateup_silu_fp8(self.xq.data_ptr(), self.xs.data_ptr(), w1q.data_ptr(), w1s.data_ptr(),
+                                               self.sorted.data_ptr(), self.eids.data_ptr(), self.npost.data_ptr(), self.M,
+                                               self.H, self.F, self.E, self.topk, p.block, self.act.data_ptr(), self.stream))
+            rec(3)
+            N.check(lib.fr_quant_e4m3_rows(self.act.data_ptr(), N.FR_BF16, p.sorted_len, self.F, self.F, self.actq.data_ptr(),
+                                           self.acts.data_ptr(), self.stream))
+            N.check(lib.fr_moe_down_combine_fp8(self.actq.data_ptr(), self.acts.data_ptr(), w2q.data_ptr(), w2s.data_ptr(),
+                                                self.tw.data_ptr(), self.sorted.data_ptr(), self.eids.data_ptr(),
+                                                self.npost.data_ptr(), self.M, self.H, self.F, self.E, self.topk, p.block,
+                                                p.split_k, N.FR_BF16, self.partial.data_ptr(), self.out.data_ptr(), self.stream))
+            rec(4)
+            return
         N.check(lib.fr_moe_gateup_silu(self.x.data_ptr(), self.w1.data_ptr(), self.sorted.data_ptr(), self.eids.data_ptr(),
                                        self.npost.data_ptr(), self.M, self.H, self.F, self.E, self.topk, p.block, N.FR_BF16,
                                        self.act.data_ptr(), self.stream))
@@ -127,14 +156,18 @@ def time_layer(torch, layer, steps, warmup):
     return wall_ms, stage_us
 
 
-def measure(torch, N, shape, M, w1, w2, steps, warmup, seed):
-    layer = Layer(torch, N, shape, M, w1, w2, seed)
+def measure(torch, N, shape, M, w1, w2, steps, warmup, seed, fp8=None):
+    layer = Layer(torch, N, shape, M, w1, w2, seed, fp8)
+    if fp8:  # pad rows of act beyond npost are never written: keep them finite for the staged quantisation
+        layer.act.zero_()
     wall_ms, stage_us = time_layer(torch, layer, steps, warmup)
     H, F, E, topk = shape["H"], shape["F"], shape["E"], shape["topk"]
     active = layer.active_experts()
-    fl, by = layer_flops(M, H, F, topk), layer_bytes(M, H, F, E, topk, active)
+    fl = layer_flops(M, H, F, topk)
+    by = layer_bytes(M, H, F, E, topk, active, bw=1 if fp8 else 2) + (active * (2 * F + H) * 4 + (M + M * topk) * 4 if fp8 else 0)
     t = wall_ms * 1e-3
-    t_hbm, t_mfma = by / (PEAK_HBM_GBS * 1e9), fl / (PEAK_BF16_TFLOPS * 1e12)
+    peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
+    t_hbm, t_mfma = by / (PEAK_HBM_GBS * 1e9), fl / (peak * 1e12)
     bound = "hbm" if t_hbm >= t_mfma else "mfma"
     rec = {
         "tokens": M, "us_per_layer": round(wall_ms * 1e3, 2), "tflops": round(fl / t / 1e12, 3),
@@ -146,17 +179,19 @@ def measure(torch, N, shape, M, w1, w2, steps, warmup, seed):
     return rec, layer
 
 
-def kernel_roofline(shape, rec):
+def kernel_roofline(shape, rec, fp8=False):
     """Roofline of the dominant kernel (gate/up grouped GEMM + SiLU*mul) from its
     event-measured average duration."""
     M, H, F, topk = rec["tokens"], shape["H"], shape["F"], shape["topk"]
     dur = rec["stage_us"]["moe_1+silu_and_mul"] * 1e-6
     flops = 4.0 * M * topk * H * F
-    byts = rec["active_experts"] * 2 * F * H * 2 + M * H * 2 + M * topk * F * 2
-    if flops / (PEAK_BF16_TFLOPS * 1e12) >= byts / (PEAK_HBM_GBS * 1e9):
+    eb = 1 if fp8 else 2
+    byts = rec["active_experts"] * 2 * F * H * eb + M * H * eb + M * topk * F * 2
+    peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
+    if flops / (peak * 1e12) >= byts / (PEAK_HBM_GBS * 1e9):
         ach = flops / dur / 1e12
-        return {"kernel": "moe_gemm_kernel<EPI_SILU>", "bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+        return {"kernel": "moe_gemm_kernel<EPI_SILU>", "bound": "mfma", "achieved": round(ach, 2), "peak": peak,
+                "unit": "TFLOP/s", "frac": round(ach / peak, 4), "traffic": None,
                 "avg_launch_us": round(dur * 1e6, 2), "algorithmic_flops_per_launch": flops}
     ach = byts / dur / 1e9
     return {"kernel": "moe_gemm_kernel<EPI_SILU>", "bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
@@ -190,6 +225,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--tokens", type=int, default=4096, help="headline token count")
     ap.add_argument("--shape", default="mixtral", choices=sorted(SHAPES))
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp8"], help="fp8: e4m3 weights + dynamic per-token activations")
     ap.add_argument("--seed", type=int, default=1337)
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
@@ -209,30 +245,36 @@ def main():
     w1 = (torch.randn(E, 2 * F, H, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
     w2 = (torch.randn(E, H, F, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
 
-    head, layer = measure(torch, N, shape, args.tokens, w1, w2, args.steps, args.warmup, args.seed)
+    fp8 = None
+    sweep_ms = shape["sweep"]
+    if args.dtype == "fp8":
+        from fast_route_amd import prepare_weights_fp8
+        fp8 = prepare_weights_fp8(w1, w2)
+        sweep_ms = [16, 256, 4096] if args.shape == "mixtral" else shape["sweep"]
+    head, layer = measure(torch, N, shape, args.tokens, w1, w2, args.steps, args.warmup, args.seed, fp8)
     sweep = []
     if not args.no_sweep:
-        for M in shape["sweep"]:
+        for M in sweep_ms:
             if M == args.tokens:
                 sweep.append(head)
                 continue
-            rec, _ = measure(torch, N, shape, M, w1, w2, args.steps, args.warmup, args.seed)
+            rec, _ = measure(torch, N, shape, M, w1, w2, args.steps, args.warmup, args.seed, fp8)
             sweep.append(rec)
     result = {
-        "metric": "moe_layer_tflops_%s_bf16_M%d" % (args.shape, args.tokens),
+        "metric": "moe_layer_tflops_%s_%s_M%d" % (args.shape, args.dtype, args.tokens),
         "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(head["us_per_layer"] / 1e3, 4), "us_per_layer": head["us_per_layer"],
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "%s-shape MoE layer: H=%d F=%d E=%d top-%d, M=%d tokens, bf16 in / fp32 accumulate"
-                               % (args.shape, H, F, E, topk, args.tokens),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "%s-shape MoE layer: H=%d F=%d E=%d top-%d, M=%d tokens, %s in / fp32 accumulate"
+                               % (args.shape, H, F, E, topk, args.tokens, args.dtype),
                    "tokens": args.tokens, "hidden": H, "ffn": F, "experts": E, "topk": topk, "seed": args.seed,
                    "flops_formula": "6*M*topk*H*F"},
         "layer_roofline_frac": head["roofline_frac"], "layer_bound": head["bound"],
         "stage_us": head["stage_us"],
-        "roofline": kernel_roofline(shape, head),
+        "roofline": kernel_roofline(shape, head, fp8 is not None),
         "sweep": sweep,
     }
-    if not args.no_cpu:
+    if not args.no_cpu and fp8 is None:
         result["cpu_baseline"] = cpu_baseline(torch, shape, layer, args.cpu_tokens)
     print(json.dumps(result))
 

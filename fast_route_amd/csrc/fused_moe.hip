@@ -58,7 +58,8 @@ int check_layer_shapes(const char* who, int64_t M, int64_t H, int64_t F, int E, 
   FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16 || dtype == FR_FP8_E4M3, FR_E_DTYPE, "%s: dtype %d not in {f16, bf16, fp8_e4m3}", who, dtype);
   FR_REQUIRE(M >= 0 && H > 0 && F > 0, FR_E_SHAPE, "%s: M=%lld H=%lld F=%lld", who, (long long)M, (long long)H, (long long)F);
   FR_REQUIRE(E >= 1 && E <= 1024 && topk >= 1 && topk <= E, FR_E_SHAPE, "%s: E=%d topk=%d", who, E, topk);
-  FR_REQUIRE(H % 128 == 0 && F % 128 == 0, FR_E_SHAPE, "%s: H=%lld and F=%lld must be multiples of 128", who, (long long)H, (long long)F);
+  const int mult = dtype == FR_FP8_E4M3 ? 256 : 128;
+  FR_REQUIRE(H % mult == 0 && F % mult == 0, FR_E_SHAPE, "%s: H=%lld and F=%lld must be multiples of %d", who, (long long)H, (long long)F, mult);
   FR_REQUIRE(M * topk < (int64_t(1) << 30), FR_E_SHAPE, "%s: M*topk too large", who);
   return FR_OK;
 }
@@ -74,19 +75,34 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   if (rc != FR_OK) return rc;
   const int64_t n = M * topk;
   const double avg = static_cast<double>(n) / E;  // expected pairs per expert under uniform load
+  // Routing block = token rows per GEMM tile.  Decode sizes want one block per expert
+  // (weights are streamed once); from ~32 pairs per expert on, the 128-row MFMA tile
+  // wins even with its padding, and 256 rows once runs are long enough to amortise it.
   int block;
   if (avg <= 8) block = 16;
-  else if (avg <= 24) block = 32;
-  else if (avg <= 64) block = 64;
+  else if (avg <= 32) block = 32;
   else if (avg <= 384) block = 128;
   else block = 256;
-  // down projection: few feature tiles (N = H), so split K until the grid covers the chip
-  const int bf = block >= 64 ? 256 : 128;
-  const int64_t active_blocks = n < E ? n : (block >= 64 ? ceil_div(n, block) + E / 2 : E);
-  const int64_t tiles = active_blocks * ceil_div(H, bf);
+  // Down projection: N = H gives few feature tiles, so K is split.
+  const int bf = block == 16 ? 64 : (block == 32 ? 128 : 256);
+  const int64_t blocks = n <= E ? n : (block >= 128 ? ceil_div(n, block) + E / 2 : E);
+  const int64_t tiles = blocks * ceil_div(H, bf);
+  const int bk_elems = dtype == FR_FP8_E4M3 ? (block <= 32 ? 256 : 128) : (block == 16 ? 128 : 64);
   int split = 1;
-  const int bk = 64;
-  while (split < 16 && tiles * split < 1024 && F / (split * 2) >= 4 * bk) split *= 2;
+  if (block >= 128) {
+    // one workgroup per CU: pick the split whose grid fills whole rounds of 256 CUs best,
+    // charging 7 % per extra fp32 partial slice (its write + re-read in the combine)
+    double best = -1.0;
+    for (int sp = 1; sp <= 4; ++sp) {
+      if (F / sp < 8 * bk_elems) break;
+      const double work = static_cast<double>(tiles) * sp;
+      const double eff = work / (256.0 * static_cast<double>(ceil_div(tiles * sp, 256))) - 0.07 * (sp - 1);
+      if (eff > best) { best = eff; split = sp; }
+    }
+  } else {
+    // several workgroups per CU: aim at ~512 workgroups
+    while (split < 16 && tiles * split * 2 <= 512 && F / (split * 2) >= 8 * bk_elems) split *= 2;
+  }
   plan->block = block;
   plan->split_k = split;
   plan->sorted_len = n + static_cast<int64_t>(E) * (block - 1);

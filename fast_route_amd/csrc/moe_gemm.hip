@@ -25,27 +25,38 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
 }
 
 // ---- host side ----------------------------------------------------------------
-// Token-block sizes and their tile shapes (K tile = 128 bytes per row everywhere).
-//   256 / 128 rows: 8 wavefronts, 32x32 MFMA, tiles streamed HBM -> LDS directly
-//                   through a 2- or 3-slot ring (compute-bound regime);
-//   64 rows:        8 wavefronts, register-staged double buffer;
-//   32 / 16 rows:   decode regime, 4 wavefronts side by side along the features,
-//                   16x16 MFMA, up to 4 workgroups per CU to keep weight bytes in flight.
-typedef Cfg<256, 256, 128, 4, 2, 32, 1, 2> CfgT256;
-typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3> CfgT128;
-typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> CfgT64;
-typedef Cfg<32, 128, 128, 1, 4, 16, 4, 0> CfgT32;
-typedef Cfg<16, 128, 128, 1, 4, 16, 4, 0> CfgT16;
-constexpr int kTileKBytes = 128;
+// Token-block sizes and their tile shapes.  K tiles are 128 bytes per row (256 for
+// the 16-row block); every block except 64 streams tiles HBM -> LDS directly.
+//   256 / 128 rows: 8 wavefronts, 32x32 MFMA, 2- or 3-slot ring (compute-bound regime);
+//   64 rows:        8 wavefronts, register-staged double buffer (op-level API only;
+//                   the fused layer goes from 32-row to 128-row blocks);
+//   32 / 16 rows:   decode regime, 16x16 MFMA, 3-slot ring, two workgroups per CU:
+//                   weight streaming at HBM rate.
+template <typename T> struct Tiles {  // bf16 / fp16
+  typedef Cfg<256, 256, 128, 4, 2, 32, 1, 2> T256;
+  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3> T128;
+  typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
+  typedef Cfg<32, 128, 128, 1, 4, 16, 2, 3> T32;
+  typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
+};
+template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per two K-steps
+  typedef Cfg<256, 256, 128, 4, 2, 32, 1, 2> T256;
+  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3> T128;
+  typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
+  typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;
+  typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
+};
 
 bool valid_block(int block) { return block == 16 || block == 32 || block == 64 || block == 128 || block == 256; }
 int elem_bytes(int dtype) { return dtype == FR_FP8_E4M3 ? 1 : 2; }
-int k_multiple(int dtype) { return kTileKBytes / elem_bytes(dtype); }
+int tile_k_bytes(int block, int dtype) { return (block == 16 || (block == 32 && dtype == FR_FP8_E4M3)) ? 256 : 128; }
+int k_multiple(int dtype, int block) { return tile_k_bytes(block, dtype) / elem_bytes(dtype); }
 
 template <typename T, int EPI>
 int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStream_t st) {
-  const int bk = kTileKBytes / static_cast<int>(sizeof(T));
-  auto fill = [&](int BT, int BF) {
+  typedef Tiles<T> TL;
+  auto fill = [&](int BT, int BF, int bkb) {
+    const int bk = bkb / static_cast<int>(sizeof(T));
     a.num_t_blocks = static_cast<int>(ceil_div(sorted_len, BT));
     const int fper = (EPI == EPI_SILU) ? BF / 2 : BF;
     a.num_f_tiles = static_cast<int>(ceil_div(a.N, fper));
@@ -53,11 +64,11 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
     a.k_per_split = static_cast<int>(round_up(ceil_div(a.K, splits), bk));
   };
   switch (block) {
-    case 256: fill(256, 256); return launch_gemm<T, CfgT256, EPI>(a, splits, st);
-    case 128: fill(128, 256); return launch_gemm<T, CfgT128, EPI>(a, splits, st);
-    case 64: fill(64, 256); return launch_gemm<T, CfgT64, EPI>(a, splits, st);
-    case 32: fill(32, 128); return launch_gemm<T, CfgT32, EPI>(a, splits, st);
-    case 16: fill(16, 128); return launch_gemm<T, CfgT16, EPI>(a, splits, st);
+    case 256: fill(256, TL::T256::BF, TL::T256::BKB); return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
+    case 128: fill(128, TL::T128::BF, TL::T128::BKB); return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
+    case 64: fill(64, TL::T64::BF, TL::T64::BKB); return launch_gemm<T, typename TL::T64, EPI>(a, splits, st);
+    case 32: fill(32, TL::T32::BF, TL::T32::BKB); return launch_gemm<T, typename TL::T32, EPI>(a, splits, st);
+    case 16: fill(16, TL::T16::BF, TL::T16::BKB); return launch_gemm<T, typename TL::T16, EPI>(a, splits, st);
     default: return fail(FR_E_SHAPE, "routing block %d not in {16, 32, 64, 128, 256}", block);
   }
 }
@@ -99,7 +110,7 @@ int gateup_impl(const void* x, const float* x_scale, const void* w1, const float
   if (M == 0) return FR_OK;
   FR_REQUIRE(x && w1 && act && sorted && expert_ids && npost, FR_E_NULL, "%s: null pointer", who);
   FR_REQUIRE(valid_block(block), FR_E_SHAPE, "%s: block=%d not in {16,32,64,128,256}", who, block);
-  FR_REQUIRE(H > 0 && H % k_multiple(dtype) == 0, FR_E_SHAPE, "%s: H=%lld must be a multiple of %d", who, (long long)H, k_multiple(dtype));
+  FR_REQUIRE(H > 0 && H % k_multiple(dtype, block) == 0, FR_E_SHAPE, "%s: H=%lld must be a multiple of %d for block %d", who, (long long)H, k_multiple(dtype, block), block);
   FR_REQUIRE(F > 0 && F % 8 == 0, FR_E_SHAPE, "%s: F=%lld must be a positive multiple of 8", who, (long long)F);
   FR_REQUIRE(topk >= 1 && E >= 1 && M * topk < (int64_t(1) << 30), FR_E_SHAPE, "%s: M*topk too large", who);
   FR_REQUIRE(aligned16(x) && aligned16(w1) && aligned16(act), FR_E_ALIGN, "%s: operands must be 16-byte aligned", who);
@@ -119,13 +130,13 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
   if (M == 0) return FR_OK;
   FR_REQUIRE(act && w2 && topk_weights && partial && out && sorted && expert_ids && npost, FR_E_NULL, "%s: null pointer", who);
   FR_REQUIRE(valid_block(block), FR_E_SHAPE, "%s: block=%d not in {16,32,64,128,256}", who, block);
-  FR_REQUIRE(F > 0 && F % k_multiple(dtype) == 0, FR_E_SHAPE, "%s: F=%lld must be a multiple of %d", who, (long long)F, k_multiple(dtype));
+  FR_REQUIRE(F > 0 && F % k_multiple(dtype, block) == 0, FR_E_SHAPE, "%s: F=%lld must be a multiple of %d for block %d", who, (long long)F, k_multiple(dtype, block), block);
   FR_REQUIRE(H > 0 && H % 4 == 0, FR_E_SHAPE, "%s: H=%lld must be a positive multiple of 4", who, (long long)H);
   FR_REQUIRE(split_k >= 1 && split_k <= 64, FR_E_SHAPE, "%s: split_k=%d outside [1, 64]", who, split_k);
   FR_REQUIRE(topk >= 1 && E >= 1 && M * topk < (int64_t(1) << 30), FR_E_SHAPE, "%s: M*topk too large", who);
   FR_REQUIRE(aligned16(act) && aligned16(w2) && aligned16(partial) && aligned16(out), FR_E_ALIGN, "%s: operands must be 16-byte aligned", who);
   const int64_t n = M * topk, sorted_len = n + int64_t(E) * (block - 1);
-  const int splits = usable_splits(split_k, F, k_multiple(dtype));
+  const int splits = usable_splits(split_k, F, k_multiple(dtype, block));
   GemmArgs a = {};
   a.X = act; a.ldx = F; a.W = w2; a.w_expert_stride = H * F; a.ldw = F; a.out = partial; a.ldo = H;
   a.split_stride = n * H;
@@ -152,7 +163,7 @@ extern "C" int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, vo
   FR_REQUIRE(!mul_routed_weight || topk_weights, FR_E_NULL, "fr_moe_grouped_gemm: mul_routed_weight without topk_weights");
   FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "fr_moe_grouped_gemm: dtype %d not in {f16, bf16}", dtype);
   FR_REQUIRE(valid_block(block), FR_E_SHAPE, "fr_moe_grouped_gemm: block=%d not in {16,32,64,128,256}", block);
-  FR_REQUIRE(K > 0 && K % k_multiple(dtype) == 0, FR_E_SHAPE, "fr_moe_grouped_gemm: K=%lld must be a positive multiple of %d", (long long)K, k_multiple(dtype));
+  FR_REQUIRE(K > 0 && K % k_multiple(dtype, block) == 0, FR_E_SHAPE, "fr_moe_grouped_gemm: K=%lld must be a positive multiple of %d for block %d", (long long)K, k_multiple(dtype, block), block);
   FR_REQUIRE(N > 0 && N % 4 == 0, FR_E_SHAPE, "fr_moe_grouped_gemm: N=%lld must be a positive multiple of 4", (long long)N);
   FR_REQUIRE(top_k >= 1 && E >= 1, FR_E_SHAPE, "fr_moe_grouped_gemm: top_k=%d E=%d", top_k, E);
   FR_REQUIRE(sorted_len >= block && sorted_len < (int64_t(1) << 31) && num_valid < (int64_t(1) << 31), FR_E_SHAPE, "fr_moe_grouped_gemm: sorted_len=%lld", (long long)sorted_len);

@@ -104,12 +104,13 @@ __device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); 
 // tile; MINB = workgroups per CU the register allocation should allow.
 // STAGES == 0: tiles go HBM -> registers -> LDS with two LDS buffers (one tile in
 // flight).  STAGES >= 2: tiles go HBM -> LDS directly (global_load_lds_dwordx4)
-// through a ring of STAGES buffers that is refilled as soon as a tile's last
-// fragments are in registers, so STAGES tiles are in flight or landed.
-template <int BT_, int BF_, int BKB_, int WT_, int WF_, int TILE_, int MINB_ = 1, int STAGES_ = 0>
+// through rings of STAGES token-tile slots and STAGES+WEXTRA weight-tile slots that
+// are refilled as soon as a tile's last fragments are in registers.
+template <int BT_, int BF_, int BKB_, int WT_, int WF_, int TILE_, int MINB_ = 1, int STAGES_ = 0, int WEXTRA_ = 0>
 struct Cfg {
   static constexpr int BT = BT_, BF = BF_, BKB = BKB_, WT = WT_, WF = WF_, TILE = TILE_, MINB = MINB_;
-  static constexpr int STAGES = STAGES_;
+  static constexpr int STAGES = STAGES_;          // ring slots of the token (X) tiles
+  static constexpr int WSTAGES = STAGES_ + WEXTRA_;  // ring slots of the weight (W) tiles: the HBM stream may run deeper
   static constexpr int NBUF = STAGES_ == 0 ? 2 : STAGES_;
   static constexpr int NT = WT * WF * kWave;       // threads
   static constexpr int NW = NT / kWave;
@@ -120,7 +121,7 @@ struct Cfg {
   static constexpr int XCH = BT * CPR, WCH = BF * CPR;
   static constexpr int XL = (XCH + NT - 1) / NT, WL = (WCH + NT - 1) / NT;
   static constexpr int XI = XCH / (kWave * NW), WI = WCH / (kWave * NW);  // direct-to-LDS loads per wave per tile
-  static constexpr int LDS_BYTES = NBUF * (BT + BF) * BKB;
+  static constexpr int LDS_BYTES = (STAGES_ == 0 ? 2 * (BT + BF) : STAGES_ * BT + (STAGES_ + WEXTRA_) * BF) * BKB;
   static_assert(TT % TILE == 0 && TF % TILE == 0, "wave tile must be a multiple of the MFMA tile");
   static_assert(NT % CPR == 0, "threads must cover whole rows");
   static_assert(STAGES_ == 0 || (STAGES_ >= 2 && XCH % (kWave * NW) == 0 && WCH % (kWave * NW) == 0),
@@ -153,7 +154,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   u32x4* lds = reinterpret_cast<u32x4*>(lds_raw);
-  constexpr int BUF = C::XCH + C::WCH;  // buffer b: X tile at b*BUF, W tile right after it
+  // LDS map (16-byte units): X slots first, then W slots
+  constexpr int NXS = C::STAGES == 0 ? 2 : C::STAGES, WBASE = NXS * C::XCH;
 
   // ---- tile coordinates ---------------------------------------------------
   // The grid is sized for the worst-case padded length; only the first
@@ -227,7 +229,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
       base = wf * C::TF + j * C::TILE;
     }
     const int r = base + frow;
-    woff[j] = C::XCH + r * CPR;
+    woff[j] = WBASE + r * CPR;
     wkey[j] = swizzle<CPR>(r, 0);
   }
 
@@ -241,15 +243,16 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
 
   // fragments, double-buffered in registers: [buffer][tile][chunk]
   u32x4 xf[2][C::IT][FC], wfr[2][C::JF][FC];
-#define FR_READ_FRAGS(stage_, ks_, fb_)                                                 \
+#define FR_READ_FRAGS(xs_, ws_, ks_, fb_)                                               \
   {                                                                                     \
-    const u32x4* tile = lds + (stage_) * BUF;                                           \
+    const u32x4* xt = lds + (xs_) * C::XCH;                                             \
+    const u32x4* wtl = lds + (ws_) * C::WCH;                                            \
     _Pragma("unroll") for (int c = 0; c < FC; ++c) {                                    \
       const int kc = ((ks_) * C::KGROUPS + kgrp) * FC + c;                              \
       _Pragma("unroll") for (int i = 0; i < C::IT; ++i)                                 \
-        xf[fb_][i][c] = tile[xoff[i] + (kc ^ xkey[i])];                                 \
+        xf[fb_][i][c] = xt[xoff[i] + (kc ^ xkey[i])];                                   \
       _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                                 \
-        wfr[fb_][j][c] = tile[woff[j] + (kc ^ wkey[j])];                                \
+        wfr[fb_][j][c] = wtl[woff[j] + (kc ^ wkey[j])];                                 \
     }                                                                                   \
   }
 #define FR_MMA(fb_, j0_, j1_)                                                           \
@@ -283,7 +286,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
       const int r = row0 + i * ROWS_PER_PASS;
       const int rr = r < BF ? r : BF - 1;
       wsrc[i] = W + static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + chunk * EPC;
-      wdst[i] = C::XCH + rr * CPR + swizzle<CPR>(rr, chunk);
+      wdst[i] = WBASE + rr * CPR + swizzle<CPR>(rr, chunk);
     }
     u32x4 xreg[C::XL], wreg[C::WL];
 #define FR_LOAD_TILE(kt)                                                              \
@@ -298,14 +301,14 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
 #define FR_STORE_TILE(buf)                                                            \
   {                                                                                   \
     _Pragma("unroll") for (int i = 0; i < C::XL; ++i)                                 \
-      if (X_FULL || row0 + i * ROWS_PER_PASS < BT) lds[(buf) * BUF + xdst[i]] = xreg[i]; \
+      if (X_FULL || row0 + i * ROWS_PER_PASS < BT) lds[(buf) * C::XCH + xdst[i]] = xreg[i]; \
     _Pragma("unroll") for (int i = 0; i < C::WL; ++i)                                 \
-      if (W_FULL || row0 + i * ROWS_PER_PASS < BF) lds[(buf) * BUF + wdst[i]] = wreg[i]; \
+      if (W_FULL || row0 + i * ROWS_PER_PASS < BF) lds[(buf) * C::WCH + wdst[i]] = wreg[i]; \
   }
 #define FR_COMPUTE_TILE(buf)                                                          \
   {                                                                                   \
     _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                               \
-      FR_READ_FRAGS(buf, ks, 0);                                                      \
+      FR_READ_FRAGS(buf, buf, ks, 0);                                                 \
       FR_MMA(0, 0, C::JF);                                                            \
     }                                                                                 \
   }
@@ -332,9 +335,9 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     // lane fetches the logical chunk that the swizzle maps to its slot.
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, LPT = XI + WI;
+    constexpr int SX = C::STAGES, SW = C::WSTAGES, NW = C::NW, XI = C::XI, WI = C::WI;
     static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
-    static_assert(S <= 5 && (S - 1) * LPT <= 63, "vmcnt budget");
+    static_assert(SW >= SX && (SX - 1) * XI + (SW - 1) * WI <= 63, "vmcnt budget");
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const T* xsrc[XI];
     const T* wsrc[WI];
@@ -350,24 +353,20 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
       wsrc[i] = W + static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * EPC;
     }
-#define FR_ISSUE_TILE(kt, stage)                                                                    \
-  {                                                                                                 \
-    unsigned char* sbase = lds_raw + (stage) * (BUF * 16);                                          \
-    _Pragma("unroll") for (int i = 0; i < XI; ++i)                                                  \
-      __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[i] + (kt) * BK),                               \
+#define FR_ISSUE_X(kt, slot_)                                                                        \
+  {                                                                                                  \
+    unsigned char* sbase = lds_raw + (slot_) * (C::XCH * 16);                                        \
+    _Pragma("unroll") for (int i = 0; i < XI; ++i)                                                   \
+      __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[i] + (kt) * BK),                                \
                                        (lptr_t)(sbase + (i * NW + wave_u) * (kWave * 16)), 16, 0, 0); \
-    _Pragma("unroll") for (int i = 0; i < WI; ++i)                                                  \
-      __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + (kt) * BK),                               \
-                                       (lptr_t)(sbase + C::XCH * 16 + (i * NW + wave_u) * (kWave * 16)), 16, 0, 0); \
   }
-    // wait until at most `tiles_after` later tiles of this lane's loads are still in flight
-    auto wait_tiles = [&](int tiles_after) {
-      if (S > 4 && tiles_after >= 4) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S > 4 ? 4 * LPT : 0) : "memory");
-      else if (S > 3 && tiles_after == 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S > 3 ? 3 * LPT : 0) : "memory");
-      else if (S > 2 && tiles_after == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S > 2 ? 2 * LPT : 0) : "memory");
-      else if (tiles_after == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
-      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    };
+#define FR_ISSUE_W(kt, slot_)                                                                        \
+  {                                                                                                  \
+    unsigned char* sbase = lds_raw + (WBASE + (slot_) * C::WCH) * 16;                                \
+    _Pragma("unroll") for (int i = 0; i < WI; ++i)                                                   \
+      __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + (kt) * BK),                                \
+                                       (lptr_t)(sbase + (i * NW + wave_u) * (kWave * 16)), 16, 0, 0); \
+  }
     // One K-step: first MFMAs of the step, then the ds_reads of the NEXT step (other
     // fragment buffer), then the remaining MFMAs, which cover the LDS latency.
     constexpr int JSPLIT = (C::JF + 1) / 2;
@@ -381,61 +380,72 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     FR_MMA(fb_, JSPLIT, C::JF);                  \
     __builtin_amdgcn_sched_barrier(0);           \
   }
-    // Software pipeline: the barrier that publishes tile kt+1 sits before the LAST
-    // K-step of tile kt, whose fragments are already in registers; the slot of tile
-    // kt is refilled right after that barrier.
+    // Software pipeline.  Loads are issued in tile order, X part before W part; the
+    // barrier that publishes tile kt+1 sits before the LAST K-step of tile kt (whose
+    // fragments are already in registers), and right after it the slots of tile kt
+    // are refilled with X(kt+SX) and W(kt+SW).  vmcnt counts loads in issue order, so
+    // "tile kt+1 landed" leaves exactly the later loads outstanding:
+    //   W(kt+1+SW-SX) of the same batch and SX-2 whole batches.
 #pragma unroll
-    for (int t = 0; t < S; ++t)
-      if (t < k_tiles) FR_ISSUE_TILE(t, t);
-    wait_tiles(min(S - 1, k_tiles - 1));
+    for (int t = 0; t < SW; ++t) {
+      if (t < SX && t < k_tiles) FR_ISSUE_X(t, t);
+      if (t < k_tiles) FR_ISSUE_W(t, t);
+    }
+    if (k_tiles >= SW) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SX - 1) * XI + (SW - 1) * WI) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
-    FR_READ_FRAGS(0, 0, 0);
+    FR_READ_FRAGS(0, 0, 0, 0);
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): no scalar load may be pending when the loop starts
-    int stage = 0;  // ring slot of tile kt
-    // steady state: tile kt+S exists, so the body is one basic block with a fixed
-    // vmcnt and the compiler can count the outstanding LDS reads exactly
+    int xs = 0, ws = 0;  // ring slots of tile kt
+    // steady state: tiles kt+SX and kt+SW exist, so the body is one basic block with a
+    // fixed vmcnt and the compiler can count the outstanding LDS reads exactly
     int kt = 0;
-    for (; kt < k_tiles - S; ++kt) {
-      const int next = (stage + 1 == S) ? 0 : stage + 1;
+    for (; kt < k_tiles - SW; ++kt) {
+      const int xn = (xs + 1 == SX) ? 0 : xs + 1, wn = (ws + 1 == SW) ? 0 : ws + 1;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         if (ks + 1 < KS) {
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(stage, ks + 1, (ks + 1) & 1));
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(xs, ws, ks + 1, (ks + 1) & 1));
         } else {
           // tile kt+1 landed (this lane's part) and this wavefront's reads of tile kt are done
-          asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((S - 2) * LPT) : "memory");
-          __builtin_amdgcn_s_barrier();  // ... everyone's: slot `stage` can be refilled
-          FR_ISSUE_TILE(kt + S, stage);
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(next, 0, 0));
+          asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(WI * (SW > SX ? 1 : 0) + (SX - 2) * (XI + WI) + (SW > SX ? 0 : 0)) : "memory");
+          __builtin_amdgcn_s_barrier();  // ... everyone's: the slots of tile kt can be refilled
+          FR_ISSUE_X(kt + SX, xs);
+          FR_ISSUE_W(kt + SW, ws);
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(xn, wn, 0, 0));
         }
       }
-      stage = next;
+      xs = xn;
+      ws = wn;
     }
-    // drain: every remaining tile is already in flight, nothing left to issue
+    // drain: no tile kt+SW any more; X tiles may still need issuing when SX < SW
     for (; kt < k_tiles - 1; ++kt) {
-      const int next = (stage + 1 == S) ? 0 : stage + 1;
+      const int xn = (xs + 1 == SX) ? 0 : xs + 1, wn = (ws + 1 == SW) ? 0 : ws + 1;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         if (ks + 1 < KS) {
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(stage, ks + 1, (ks + 1) & 1));
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(xs, ws, ks + 1, (ks + 1) & 1));
         } else {
-          wait_tiles(k_tiles - 2 - kt);
+          asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
           __builtin_amdgcn_s_barrier();
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(next, 0, 0));
+          if (kt + SX < k_tiles) FR_ISSUE_X(kt + SX, xs);
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(xn, wn, 0, 0));
         }
       }
-      stage = next;
+      xs = xn;
+      ws = wn;
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {  // last tile
       if (ks + 1 < KS) {
-        FR_KSTEP(ks & 1, FR_READ_FRAGS(stage, ks + 1, (ks + 1) & 1));
+        FR_KSTEP(ks & 1, FR_READ_FRAGS(xs, ws, ks + 1, (ks + 1) & 1));
       } else {
         FR_KSTEP(ks & 1, {});
       }
     }
 #undef FR_KSTEP
-#undef FR_ISSUE_TILE
+#undef FR_ISSUE_X
+#undef FR_ISSUE_W
   }
 #undef FR_READ_FRAGS
 #undef FR_MMA
