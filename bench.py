@@ -218,6 +218,57 @@ def cpu_baseline(torch, shape, layer, sample_tokens):
             "ref_max_abs": ref.abs().max().item()}
 
 
+def routing_bench(torch, N, steps, warmup, seed):
+    """Routing-only stress workload: 65536 tokens, 64 experts, top-6, Zipf(1.2)-skewed
+    logits; gating + block-aligned sort for block in {16, 32, 64, 128}, checked bit-exact
+    against the CPU oracle once, then timed."""
+    import numpy as np
+    import oracle
+    M, E, k = 65536, 64, 6
+    logits = oracle.zipf_logits(M, E, seed)
+    dl = logits.cuda()
+    n = M * k
+    tw = torch.empty(n, dtype=torch.float32, device="cuda")
+    ti = torch.empty(n, dtype=torch.int32, device="cuda")
+    lib, st = N.lib(), torch.cuda.current_stream().cuda_stream
+    ws_bytes = lib.fr_moe_align_workspace_bytes(n, E)
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device="cuda")
+    _, ref_ids = oracle.gating_topk(logits, k, True)
+    out = []
+    for B in (16, 32, 64, 128):
+        sl = n + E * (B - 1)
+        s_ = torch.empty(sl, dtype=torch.int32, device="cuda")
+        e_ = torch.empty(n + E, dtype=torch.int32, device="cuda")
+        p_ = torch.empty(1, dtype=torch.int32, device="cuda")
+
+        def gate():
+            N.check(lib.fr_gating_topk(dl.data_ptr(), N.FR_F32, M, E, E, k, 1, tw.data_ptr(), ti.data_ptr(), st))
+
+        def align():
+            N.check(lib.fr_moe_align(ti.data_ptr(), N.FR_I32, n, E, B, s_.data_ptr(), e_.data_ptr(), p_.data_ptr(),
+                                     ws.data_ptr(), ws_bytes, st))
+        gate(); align(); torch.cuda.synchronize()
+        rs, re_, rn = oracle.moe_align_block_size(ref_ids, B, E)
+        exact = bool(torch.equal(ti.cpu().view(M, k), ref_ids) and np.array_equal(s_.cpu().numpy(), rs)
+                     and int(p_.cpu()[0]) == int(rn[0]))
+        for _ in range(warmup):
+            gate(); align()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        tg = ta = 0.0
+        for _ in range(steps):
+            ev[0].record(); gate(); ev[1].record(); align(); ev[2].record()
+            torch.cuda.synchronize()
+            tg += ev[0].elapsed_time(ev[1]); ta += ev[1].elapsed_time(ev[2])
+        npost = int(p_.cpu()[0])
+        a_bytes = 4 * n + 4 * npost + 4 * (npost // B) + 4
+        g_bytes = M * E * 4 + 8 * n
+        out.append({"block": B, "bit_exact": exact, "gating_us": round(tg * 1e3 / steps, 2),
+                    "align_us": round(ta * 1e3 / steps, 2), "align_ns_per_pair": round(ta * 1e6 / steps / n, 4),
+                    "align_gbps": round(a_bytes / (ta * 1e-3 / steps) / 1e9, 2),
+                    "gating_gbps": round(g_bytes / (tg * 1e-3 / steps) / 1e9, 1), "npost": npost})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -230,6 +281,7 @@ def main():
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=1024)
+    ap.add_argument("--routing", action="store_true", help="also time the routing-only stress workload")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X runs the whole layer); --gpus must be 1")
@@ -274,6 +326,8 @@ def main():
         "roofline": kernel_roofline(shape, head, fp8 is not None),
         "sweep": sweep,
     }
+    if args.routing:
+        result["routing_stress"] = routing_bench(torch, N, args.steps, args.warmup, args.seed)
     if not args.no_cpu and fp8 is None:
         result["cpu_baseline"] = cpu_baseline(torch, shape, layer, args.cpu_tokens)
     print(json.dumps(result))

@@ -49,13 +49,15 @@ constexpr int kWave = 64;
 // partner<S>(v): value held by this lane's partner at butterfly step S.  Steps
 // 1 and 2 are DPP quad permutes, 4 and 8 DPP mirrors inside a row of 16 lanes
 // (an involution that pairs the two halves, which is all an all-reduce needs),
-// 16 and 32 go through the LDS crossbar.
+// 16 and 32 go through the LDS crossbar.  All lanes are written (full row/bank masks,
+// every source lane valid), so `old` is a don't-care; passing 0 with bound_ctrl lets
+// the compiler fold the move into the consuming VALU instruction.
 template <int S>
 __device__ __forceinline__ int partner_i32(int v) {
-  if constexpr (S == 1) return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
-  else if constexpr (S == 2) return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
-  else if constexpr (S == 4) return __builtin_amdgcn_update_dpp(v, v, 0x141, 0xF, 0xF, false); // row_half_mirror
-  else if constexpr (S == 8) return __builtin_amdgcn_update_dpp(v, v, 0x140, 0xF, 0xF, false); // row_mirror
+  if constexpr (S == 1) return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+  else if constexpr (S == 2) return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+  else if constexpr (S == 4) return __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true); // row_half_mirror
+  else if constexpr (S == 8) return __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true); // row_mirror
   else return __shfl_xor(v, S, kWave);
 }
 template <int S>

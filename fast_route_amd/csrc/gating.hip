@@ -20,27 +20,80 @@ __device__ __forceinline__ bool better(float av, int ai, float bv, int bi) {
   return av > bv || (av == bv && ai < bi);
 }
 
+// max over the group, returned in every lane: DPP steps inside a row of 16 lanes,
+// then the (uniform per row) row maxima are read out as scalars and combined
+template <int G>
+__device__ __forceinline__ float group_max(float v) {
+  if constexpr (G > 1) v = fmaxf(v, partner_f32<1>(v));
+  if constexpr (G > 2) v = fmaxf(v, partner_f32<2>(v));
+  if constexpr (G > 4) v = fmaxf(v, partner_f32<4>(v));
+  if constexpr (G > 8) v = fmaxf(v, partner_f32<8>(v));
+  if constexpr (G > 16) {
+    const int bits = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(bits, 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(bits, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(bits, 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(bits, 48));
+    if constexpr (G == 32) v = (threadIdx.x & 32) ? fmaxf(r2, r3) : fmaxf(r0, r1);
+    else v = fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+  }
+  return v;
+}
+
+// sum over the group, same scheme (every lane adds the same numbers in the same order)
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+  if constexpr (G > 1) v += partner_f32<1>(v);
+  if constexpr (G > 2) v += partner_f32<2>(v);
+  if constexpr (G > 4) v += partner_f32<4>(v);
+  if constexpr (G > 8) v += partner_f32<8>(v);
+  if constexpr (G > 16) {
+    const int bits = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(bits, 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(bits, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(bits, 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(bits, 48));
+    if constexpr (G == 32) v = (threadIdx.x & 32) ? (r2 + r3) : (r0 + r1);
+    else v = (r0 + r1) + (r2 + r3);
+  }
+  return v;
+}
+
+// Order-preserving map fp32 -> uint32 (larger float <=> larger key; every real value,
+// -inf included, maps above 0, which serves as "not a candidate").
+__device__ __forceinline__ unsigned float_key(float v) {
+  const unsigned b = __float_as_uint(v);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float key_float(unsigned k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7FFFFFFFu) : ~k);
+}
+// unsigned max over the group, in every lane (integer max needs no NaN canonicalisation,
+// so the DPP moves fold into v_max_u32; rows are combined on the scalar unit)
+template <int G>
+__device__ __forceinline__ unsigned group_max_key(unsigned k) {
+  if constexpr (G > 1) k = max(k, static_cast<unsigned>(partner_i32<1>(static_cast<int>(k))));
+  if constexpr (G > 2) k = max(k, static_cast<unsigned>(partner_i32<2>(static_cast<int>(k))));
+  if constexpr (G > 4) k = max(k, static_cast<unsigned>(partner_i32<4>(static_cast<int>(k))));
+  if constexpr (G > 8) k = max(k, static_cast<unsigned>(partner_i32<8>(static_cast<int>(k))));
+  if constexpr (G > 16) {
+    const unsigned r0 = __builtin_amdgcn_readlane(static_cast<int>(k), 0);
+    const unsigned r1 = __builtin_amdgcn_readlane(static_cast<int>(k), 16);
+    const unsigned r2 = __builtin_amdgcn_readlane(static_cast<int>(k), 32);
+    const unsigned r3 = __builtin_amdgcn_readlane(static_cast<int>(k), 48);
+    if constexpr (G == 32) k = (threadIdx.x & 32) ? max(r2, r3) : max(r0, r1);
+    else k = max(max(r0, r1), max(r2, r3));
+  }
+  return k;
+}
+
+// Cross-lane merge of per-lane online-softmax states (m = running max, s = sum of
+// exp(x - m)): one max reduction, one rescale, one sum reduction.
 template <int G>
 __device__ __forceinline__ void group_online_softmax(float& m, float& s) {
-  auto step = [&](auto tag) {
-    constexpr int S = decltype(tag)::value;
-    const float m2 = partner_f32<S>(m);
-    const float s2 = partner_f32<S>(s);
-    const float mn = fmaxf(m, m2);
-    const float a = (m == -INFINITY) ? 0.f : s * expf(m - mn);
-    const float b = (m2 == -INFINITY) ? 0.f : s2 * expf(m2 - mn);
-    // a + b is evaluated with the lower lane's term first in both partners so
-    // every lane of the group ends with bit-identical statistics
-    const bool low = (static_cast<int>(threadIdx.x) & S) == 0;
-    s = low ? (a + b) : (b + a);
-    m = mn;
-  };
-  if constexpr (G > 1) step(std::integral_constant<int, 1>{});
-  if constexpr (G > 2) step(std::integral_constant<int, 2>{});
-  if constexpr (G > 4) step(std::integral_constant<int, 4>{});
-  if constexpr (G > 8) step(std::integral_constant<int, 8>{});
-  if constexpr (G > 16) step(std::integral_constant<int, 16>{});
-  if constexpr (G > 32) step(std::integral_constant<int, 32>{});
+  const float gm = group_max<G>(m);
+  s = group_sum<G>((m == -INFINITY) ? 0.f : s * __expf(m - gm));
+  m = gm;
 }
 
 template <int G>
@@ -77,13 +130,17 @@ __device__ __forceinline__ void gate_token(Load load, bool live, int E, int topk
     v[i] = (live && e < E) ? load(e) : -INFINITY;
   }
 
-  // online softmax statistics over this lane's values, then across the group
+  // online softmax over this lane's values (running max, rescaled running sum),
+  // then merged across the group
   float m = v[0];
+  float s = (v[0] == -INFINITY) ? 0.f : 1.f;
 #pragma unroll
-  for (int i = 1; i < VPL; ++i) m = fmaxf(m, v[i]);
-  float s = 0.f;
-#pragma unroll
-  for (int i = 0; i < VPL; ++i) s += (v[i] == -INFINITY) ? 0.f : expf(v[i] - m);
+  for (int i = 1; i < VPL; ++i) {
+    if (v[i] == -INFINITY) continue;
+    const float mn = fmaxf(m, v[i]);
+    s = (m == -INFINITY ? 0.f : s * __expf(m - mn)) + __expf(v[i] - mn);
+    m = mn;
+  }
   group_online_softmax<G>(m, s);
 
   float sel_v[VPL];
@@ -95,20 +152,35 @@ __device__ __forceinline__ void gate_token(Load load, bool live, int E, int topk
   }
   unsigned taken = 0;
   float sel_sum = 0.f;
+  const unsigned vkey = float_key(v[0]);
   for (int r = 0; r < topk; ++r) {
-    float bv = -INFINITY;
-    int bi = INT_MAX;
+    float bv;
+    int bi;
+    if constexpr (VPL == 1) {
+      // one logit per lane, lane order = expert order: the winner is the group max and,
+      // among lanes holding it, the lowest lane (= lowest expert index) of a ballot
+      const unsigned key = (g < E && !taken) ? vkey : 0u;
+      const unsigned top = group_max_key<G>(key);
+      bv = key_float(top);
+      unsigned long long hit = __ballot(key == top);
+      if constexpr (G < 64) hit = (hit >> (threadIdx.x & 63 & ~(G - 1))) & ((1ull << G) - 1ull);
+      bi = __ffsll(hit) - 1;
+      if (bi == g) taken = 1u;
+    } else {
+      bv = -INFINITY;
+      bi = INT_MAX;
 #pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-      const int e = g + i * G;
-      if (e < E && !((taken >> i) & 1u) && better(v[i], e, bv, bi)) {
-        bv = v[i];
-        bi = e;
+      for (int i = 0; i < VPL; ++i) {
+        const int e = g + i * G;
+        if (e < E && !((taken >> i) & 1u) && better(v[i], e, bv, bi)) {
+          bv = v[i];
+          bi = e;
+        }
       }
+      group_argmax<G>(bv, bi);
+      if (bi % G == g) taken |= 1u << (bi / G);
     }
-    group_argmax<G>(bv, bi);
-    if (bi % G == g) taken |= 1u << (bi / G);
-    sel_sum += expf(bv - m);
+    sel_sum += __expf(bv - m);
 #pragma unroll
     for (int sl = 0; sl < VPL; ++sl) {
       if (r == sl * G + g) {
@@ -124,7 +196,7 @@ __device__ __forceinline__ void gate_token(Load load, bool live, int E, int topk
     for (int sl = 0; sl < VPL; ++sl) {
       const int r = sl * G + g;
       if (r < topk) {
-        w_row[r] = expf(sel_v[sl] - m) / denom;
+        w_row[r] = __expf(sel_v[sl] - m) / denom;
         id_row[r] = sel_i[sl];
       }
     }
@@ -135,11 +207,17 @@ template <typename T, int G, int VPL>
 __global__ __launch_bounds__(kGateThreads) void gating_topk_kernel(
     const T* __restrict__ logits, int64_t M, int E, int64_t ld, int topk, int renorm,
     float* __restrict__ w_out, int32_t* __restrict__ ids_out) {
-  const int64_t token = (static_cast<int64_t>(blockIdx.x) * kGateThreads + threadIdx.x) / G;
-  const bool live = token < M;
-  const T* row = logits + (live ? token : 0) * ld;
-  gate_token<G, VPL>([&](int e) { return to_float(row[e]); }, live, E, topk, renorm,
-                     w_out + token * topk, ids_out + token * topk);
+  // grid-stride over tokens: a few tokens per lane group amortise wave launch
+  constexpr int64_t kPerBlock = kGateThreads / G;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kPerBlock;
+  const int64_t rounds = (M + stride - 1) / stride;  // uniform trip count: every lane joins the cross-lane ops
+  int64_t token = static_cast<int64_t>(blockIdx.x) * kPerBlock + threadIdx.x / G;
+  for (int64_t it = 0; it < rounds; ++it, token += stride) {
+    const bool live = token < M;
+    const T* row = logits + (live ? token : 0) * ld;
+    gate_token<G, VPL>([&](int e) { return to_float(row[e]); }, live, E, topk, renorm,
+                       w_out + token * topk, ids_out + token * topk);
+  }
 }
 
 // ---- gate-matrix form: logits tile by MFMA, then the same gating -------------
@@ -228,7 +306,9 @@ template <typename T, int G, int VPL>
 void launch(const void* logits, int64_t M, int E, int64_t ld, int topk, int renorm, float* w,
             int32_t* ids, hipStream_t st) {
   const int64_t tokens_per_block = kGateThreads / G;
-  const unsigned grid = static_cast<unsigned>(ceil_div(M, tokens_per_block));
+  int64_t blocks = ceil_div(M, tokens_per_block);
+  if (blocks > 4096) blocks = 4096;  // 16 workgroups per CU; the rest is the in-kernel token loop
+  const unsigned grid = static_cast<unsigned>(blocks);
   hipLaunchKernelGGL((gating_topk_kernel<T, G, VPL>), dim3(grid), dim3(kGateThreads), 0, st,
                      static_cast<const T*>(logits), M, E, ld, topk, renorm, w, ids);
 }

@@ -8,7 +8,8 @@
 // 64 pairs at a time and ranks the pairs of one expert among themselves with
 // wavefront ballots, so flat order survives inside each expert: the result is
 // the stable sort.  Small inputs run all three phases in one workgroup with the
-// tables in LDS; large ones use three launches and a global table.
+// tables in LDS; large ones use three launches (count, per-expert segment scan,
+// scatter + block table) and a global table.
 #include "fr_common.h"
 
 namespace fr {
@@ -21,8 +22,6 @@ constexpr int64_t kSmallMaxN = 16384;
 constexpr int kMaxE = 1024;
 constexpr int kSegThreads = 256;
 constexpr int kSegWaves = kSegThreads / kWave;
-constexpr int kScanThreads = 1024;
-constexpr int kScanWaves = kScanThreads / kWave;
 
 __device__ __forceinline__ int64_t min64(int64_t a, int64_t b) { return a < b ? a : b; }
 
@@ -158,8 +157,8 @@ __global__ __launch_bounds__(kSmallThreads) void align_small_kernel(
 }
 
 // ---------------------------------------------------------------- large path
-// counts is [E][S]: after align_scan_kernel, counts[e][s] is the offset of
-// segment s inside expert e's run and run_start[e] the start of the run.
+// counts is [E][S]: after align_segscan_kernel, counts[e][s] is the offset of
+// segment s inside expert e's run and totals[e] the length of the run.
 template <typename IdT>
 __global__ __launch_bounds__(kSegThreads) void align_count_kernel(
     const IdT* __restrict__ ids, int64_t n, int E, int seg_len, int S, int* __restrict__ counts) {
@@ -177,42 +176,60 @@ __global__ __launch_bounds__(kSegThreads) void align_count_kernel(
   for (int e = lane; e < E; e += kWave) counts[static_cast<int64_t>(e) * S + seg] = mine[e];
 }
 
-__global__ __launch_bounds__(kScanThreads) void align_scan_kernel(
-    int* __restrict__ counts, int* __restrict__ run_start, int64_t n, int E, int B, int S,
-    int64_t sorted_len, int32_t* __restrict__ sorted, int32_t* __restrict__ expert_ids,
-    int32_t* __restrict__ npost_out) {
-  __shared__ int total[kMaxE];
-  __shared__ int start[kMaxE + 1];
-  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  for (int e = wave; e < E; e += kScanWaves) {
-    int* row = counts + static_cast<int64_t>(e) * S;
-    int running = 0;
-    for (int base = 0; base < S; base += kWave) {
-      const int s = base + lane;
-      const int c = (s < S) ? row[s] : 0;
-      const int incl = wave_inclusive_scan(c, lane);
-      if (s < S) row[s] = running + incl - c;
-      running += __shfl(incl, kWave - 1, kWave);
+// One workgroup per expert: exclusive scan of that expert's per-segment counts
+// (in place) and its total.
+__global__ __launch_bounds__(kSegThreads) void align_segscan_kernel(int* __restrict__ counts,
+                                                                     int* __restrict__ totals, int S) {
+  __shared__ int wave_sum[kSegWaves];
+  const int e = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  int* row = counts + static_cast<int64_t>(e) * S;
+  int running = 0;
+  for (int base = 0; base < S; base += kSegThreads) {
+    const int s = base + tid;
+    const int c = (s < S) ? row[s] : 0;
+    const int incl = wave_inclusive_scan(c, lane);
+    if (lane == kWave - 1) wave_sum[wave] = incl;
+    __syncthreads();
+    int before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < kSegWaves; ++w) {
+      const int ws = wave_sum[w];
+      before += (w < wave) ? ws : 0;
+      all += ws;
     }
-    if (lane == 0) total[e] = running;
+    if (s < S) row[s] = running + before + incl - c;
+    running += all;
+    __syncthreads();
   }
-  __syncthreads();
-  if (wave == 0) scan_padded_totals(total, start, E, B, lane);
-  __syncthreads();
-  for (int e = tid; e < E; e += kScanThreads) run_start[e] = start[e];
-  write_block_table(total, start, E, B, n, sorted_len, tid, kScanThreads, sorted, expert_ids, npost_out);
+  if (tid == 0) totals[e] = running;
 }
 
+// Scatter pass.  Every workgroup rebuilds the run starts from the E totals (cheap),
+// workgroup e < E also writes expert e's block table and padding, workgroup 0 the
+// tail and the padded length; then each wavefront places its segment.
 template <typename IdT>
 __global__ __launch_bounds__(kSegThreads) void align_scatter_kernel(
-    const IdT* __restrict__ ids, int64_t n, int E, int seg_len, int S, const int* __restrict__ counts,
-    const int* __restrict__ run_start, int32_t* __restrict__ sorted) {
+    const IdT* __restrict__ ids, int64_t n, int E, int B, int seg_len, int S, int64_t sorted_len,
+    const int* __restrict__ counts, const int* __restrict__ totals, int32_t* __restrict__ sorted,
+    int32_t* __restrict__ expert_ids, int32_t* __restrict__ npost_out) {
   extern __shared__ int hist[];  // [kSegWaves][E]
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  __shared__ int start[kMaxE + 1];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  if (wave == 0) scan_padded_totals(totals, start, E, B, lane);
+  __syncthreads();
+  if (static_cast<int>(blockIdx.x) < E) {
+    const int e = blockIdx.x;
+    for (int b = start[e] / B + tid; b < start[e + 1] / B; b += kSegThreads) expert_ids[b] = e;
+    for (int s = start[e] + totals[e] + tid; s < start[e + 1]; s += kSegThreads) sorted[s] = static_cast<int32_t>(n);
+  }
+  if (blockIdx.x == 0) {
+    for (int64_t s = start[E] + tid; s < sorted_len; s += kSegThreads) sorted[s] = static_cast<int32_t>(n);
+    if (tid == 0) npost_out[0] = start[E];
+  }
   const int seg = blockIdx.x * kSegWaves + wave;
   if (seg >= S) return;
   int* mine = hist + wave * E;
-  for (int e = lane; e < E; e += kWave) mine[e] = run_start[e] + counts[static_cast<int64_t>(e) * S + seg];
+  for (int e = lane; e < E; e += kWave) mine[e] = start[e] + counts[static_cast<int64_t>(e) * S + seg];
   __builtin_amdgcn_wave_barrier();
   const int64_t lo = static_cast<int64_t>(seg) * seg_len;
   const int64_t hi = min64(n, lo + seg_len);
@@ -243,13 +260,13 @@ int run(const void* ids_v, int64_t n, int E, int B, int32_t* sorted, int32_t* ex
   int* counts = static_cast<int*>(ws);
   int* run_start = counts + static_cast<int64_t>(E) * S;
   const unsigned blocks = static_cast<unsigned>(ceil_div(S, kSegWaves));
+  const unsigned scatter_blocks = blocks > static_cast<unsigned>(E) ? blocks : static_cast<unsigned>(E);
   const size_t lds = sizeof(int) * kSegWaves * E;
   hipLaunchKernelGGL((align_count_kernel<IdT>), dim3(blocks), dim3(kSegThreads), lds, st, ids, n, E,
                      seg_len, S, counts);
-  hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, counts, run_start, n, E, B, S,
-                     sorted_len, sorted, expert_ids, npost);
-  hipLaunchKernelGGL((align_scatter_kernel<IdT>), dim3(blocks), dim3(kSegThreads), lds, st, ids, n, E,
-                     seg_len, S, counts, run_start, sorted);
+  hipLaunchKernelGGL(align_segscan_kernel, dim3(E), dim3(kSegThreads), 0, st, counts, run_start, S);
+  hipLaunchKernelGGL((align_scatter_kernel<IdT>), dim3(scatter_blocks), dim3(kSegThreads), lds, st, ids, n, E, B,
+                     seg_len, S, sorted_len, counts, run_start, sorted, expert_ids, npost);
   return check_launch("align kernels");
 }
 
