@@ -104,13 +104,13 @@ __device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); 
 // tile; MINB = workgroups per CU the register allocation should allow.
 // STAGES == 0: tiles go HBM -> registers -> LDS with two LDS buffers (one tile in
 // flight).  STAGES >= 2: tiles go HBM -> LDS directly (global_load_lds_dwordx4)
-// through rings of STAGES token-tile slots and STAGES+WEXTRA weight-tile slots that
-// are refilled as soon as a tile's last fragments are in registers.
-template <int BT_, int BF_, int BKB_, int WT_, int WF_, int TILE_, int MINB_ = 1, int STAGES_ = 0, int WEXTRA_ = 0>
+// through rings of STAGES token-tile and weight-tile slots; a slot is refilled once
+// its tile's last fragments are in registers, the loads spread over SPREAD K-steps.
+template <int BT_, int BF_, int BKB_, int WT_, int WF_, int TILE_, int MINB_ = 1, int STAGES_ = 0, int SPREAD_ = 0>
 struct Cfg {
   static constexpr int BT = BT_, BF = BF_, BKB = BKB_, WT = WT_, WF = WF_, TILE = TILE_, MINB = MINB_;
-  static constexpr int STAGES = STAGES_;          // ring slots of the token (X) tiles
-  static constexpr int WSTAGES = STAGES_ + WEXTRA_;  // ring slots of the weight (W) tiles: the HBM stream may run deeper
+  static constexpr int STAGES = STAGES_;  // ring slots of the token and of the weight tiles
+  static constexpr int SPREAD = SPREAD_;  // K-steps over which the refill of a slot is spread (<= 1: one burst)
   static constexpr int NBUF = STAGES_ == 0 ? 2 : STAGES_;
   static constexpr int NT = WT * WF * kWave;       // threads
   static constexpr int NW = NT / kWave;
@@ -121,7 +121,7 @@ struct Cfg {
   static constexpr int XCH = BT * CPR, WCH = BF * CPR;
   static constexpr int XL = (XCH + NT - 1) / NT, WL = (WCH + NT - 1) / NT;
   static constexpr int XI = XCH / (kWave * NW), WI = WCH / (kWave * NW);  // direct-to-LDS loads per wave per tile
-  static constexpr int LDS_BYTES = (STAGES_ == 0 ? 2 * (BT + BF) : STAGES_ * BT + (STAGES_ + WEXTRA_) * BF) * BKB;
+  static constexpr int LDS_BYTES = (STAGES_ == 0 ? 2 : STAGES_) * (BT + BF) * BKB;
   static_assert(TT % TILE == 0 && TF % TILE == 0, "wave tile must be a multiple of the MFMA tile");
   static_assert(NT % CPR == 0, "threads must cover whole rows");
   static_assert(STAGES_ == 0 || (STAGES_ >= 2 && XCH % (kWave * NW) == 0 && WCH % (kWave * NW) == 0),
@@ -335,9 +335,13 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     // lane fetches the logical chunk that the swizzle maps to its slot.
     typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    constexpr int SX = C::STAGES, SW = C::WSTAGES, NW = C::NW, XI = C::XI, WI = C::WI;
+    constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, NL = XI + WI;
+    // The NL loads that refill a slot are issued in PARTS groups of PER, one group per
+    // K-step, so the data does not arrive at the LDS in one burst that starves ds_read.
+    constexpr int PARTS = C::SPREAD < 1 ? 1 : (C::SPREAD > KS - 1 ? (KS > 1 ? KS - 1 : 1) : C::SPREAD);
+    constexpr int PER = (NL + PARTS - 1) / PARTS, P0 = PER < NL ? PER : NL;
     static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
-    static_assert(SW >= SX && (SX - 1) * XI + (SW - 1) * WI <= 63, "vmcnt budget");
+    static_assert((S - 1) * NL <= 63, "vmcnt budget");
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const T* xsrc[XI];
     const T* wsrc[WI];
@@ -353,99 +357,107 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
       wsrc[i] = W + static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * EPC;
     }
-#define FR_ISSUE_X(kt, slot_)                                                                        \
-  {                                                                                                  \
-    unsigned char* sbase = lds_raw + (slot_) * (C::XCH * 16);                                        \
-    _Pragma("unroll") for (int i = 0; i < XI; ++i)                                                   \
-      __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[i] + (kt) * BK),                                \
-                                       (lptr_t)(sbase + (i * NW + wave_u) * (kWave * 16)), 16, 0, 0); \
+    // group p_ of the loads of tile tile_ into ring slot slot_: token-tile loads first
+#define FR_ISSUE_PART(tile_, slot_, p_)                                                                    \
+  {                                                                                                        \
+    _Pragma("unroll") for (int q = (p_) * PER; q < ((p_) + 1) * PER && q < NL; ++q) {                      \
+      if (q < XI) {                                                                                        \
+        __builtin_amdgcn_global_load_lds(                                                                  \
+            (gptr_t)(xsrc[q < XI ? q : 0] + (tile_) * BK),                                                 \
+            (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + (q * NW + wave_u) * (kWave * 16)), 16, 0, 0);     \
+      } else {                                                                                             \
+        __builtin_amdgcn_global_load_lds(                                                                  \
+            (gptr_t)(wsrc[q < XI ? 0 : q - XI] + (tile_) * BK),                                            \
+            (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + ((q - XI) * NW + wave_u) * (kWave * 16)), \
+            16, 0, 0);                                                                                     \
+      }                                                                                                    \
+    }                                                                                                      \
   }
-#define FR_ISSUE_W(kt, slot_)                                                                        \
-  {                                                                                                  \
-    unsigned char* sbase = lds_raw + (WBASE + (slot_) * C::WCH) * 16;                                \
-    _Pragma("unroll") for (int i = 0; i < WI; ++i)                                                   \
-      __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + (kt) * BK),                                \
-                                       (lptr_t)(sbase + (i * NW + wave_u) * (kWave * 16)), 16, 0, 0); \
-  }
-    // One K-step: first MFMAs of the step, then the ds_reads of the NEXT step (other
-    // fragment buffer), then the remaining MFMAs, which cover the LDS latency.
+    // One K-step: the first half of the MFMAs covers the LDS latency of the fragments
+    // of the NEXT step, which are read into the other fragment buffer; a group of
+    // refill loads, if any, goes out between the halves.
     constexpr int JSPLIT = (C::JF + 1) / 2;
-#define FR_KSTEP(fb_, READ_NEXT)                 \
+#define FR_KSTEP(fb_, READ_NEXT, ISSUE)          \
   {                                              \
-    __builtin_amdgcn_sched_barrier(0);           \
     FR_MMA(fb_, 0, JSPLIT);                      \
     __builtin_amdgcn_sched_barrier(0);           \
     READ_NEXT;                                   \
+    ISSUE;                                       \
     __builtin_amdgcn_sched_barrier(0);           \
     FR_MMA(fb_, JSPLIT, C::JF);                  \
     __builtin_amdgcn_sched_barrier(0);           \
   }
-    // Software pipeline.  Loads are issued in tile order, X part before W part; the
-    // barrier that publishes tile kt+1 sits before the LAST K-step of tile kt (whose
-    // fragments are already in registers), and right after it the slots of tile kt
-    // are refilled with X(kt+SX) and W(kt+SW).  vmcnt counts loads in issue order, so
-    // "tile kt+1 landed" leaves exactly the later loads outstanding:
-    //   W(kt+1+SW-SX) of the same batch and SX-2 whole batches.
+    // Software pipeline.  Tiles are loaded in order; the barrier that publishes tile
+    // kt+1 sits before the LAST K-step of tile kt (whose fragments are already in
+    // registers).  After it the slot of tile kt is refilled with tile kt+S: group 0 in
+    // that last K-step, groups 1.. in the first K-steps of tile kt+1.  vmcnt counts
+    // loads in issue order, so "tile kt+1 landed" leaves exactly the S-2 later tiles
+    // outstanding.  The prologue leaves tile S-1 in the same half-issued state.
 #pragma unroll
-    for (int t = 0; t < SW; ++t) {
-      if (t < SX && t < k_tiles) FR_ISSUE_X(t, t);
-      if (t < k_tiles) FR_ISSUE_W(t, t);
+    for (int t = 0; t < S; ++t) {
+      if (t < k_tiles) {
+        FR_ISSUE_PART(t, t, 0);
+        if (t < S - 1) {
+#pragma unroll
+          for (int p = 1; p < PARTS; ++p) FR_ISSUE_PART(t, t, p);
+        }
+      }
     }
-    if (k_tiles >= SW) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SX - 1) * XI + (SW - 1) * WI) : "memory");
+    if (k_tiles >= S) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((S - 2) * NL + P0) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     FR_READ_FRAGS(0, 0, 0, 0);
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): no scalar load may be pending when the loop starts
-    int xs = 0, ws = 0;  // ring slots of tile kt
-    // steady state: tiles kt+SX and kt+SW exist, so the body is one basic block with a
-    // fixed vmcnt and the compiler can count the outstanding LDS reads exactly
+    int sl = 0;  // ring slot of tile kt
+    // steady state: tile kt+S exists, so the body is one basic block with a fixed vmcnt
+    // and the compiler can count the outstanding LDS reads exactly
     int kt = 0;
-    for (; kt < k_tiles - SW; ++kt) {
-      const int xn = (xs + 1 == SX) ? 0 : xs + 1, wn = (ws + 1 == SW) ? 0 : ws + 1;
+    for (; kt < k_tiles - S; ++kt) {
+      const int sn = (sl + 1 == S) ? 0 : sl + 1, sp = (sl == 0) ? S - 1 : sl - 1;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         if (ks + 1 < KS) {
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(xs, ws, ks + 1, (ks + 1) & 1));
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1),
+                   if (ks + 1 < PARTS) FR_ISSUE_PART(kt - 1 + S, sp, ks + 1));
         } else {
           // tile kt+1 landed (this lane's part) and this wavefront's reads of tile kt are done
-          asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(WI * (SW > SX ? 1 : 0) + (SX - 2) * (XI + WI) + (SW > SX ? 0 : 0)) : "memory");
-          __builtin_amdgcn_s_barrier();  // ... everyone's: the slots of tile kt can be refilled
-          FR_ISSUE_X(kt + SX, xs);
-          FR_ISSUE_W(kt + SW, ws);
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(xn, wn, 0, 0));
+          asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((S - 2) * NL) : "memory");
+          __builtin_amdgcn_s_barrier();  // ... everyone's: the slot of tile kt can be refilled
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, sn, 0, 0), FR_ISSUE_PART(kt + S, sl, 0));
         }
       }
-      xs = xn;
-      ws = wn;
+      sl = sn;
     }
-    // drain: no tile kt+SW any more; X tiles may still need issuing when SX < SW
+    // drain: finish the half-issued refill (the last tile), then no more loads
+    if (k_tiles >= S) {
+      const int sp = (sl == 0) ? S - 1 : sl - 1;
+#pragma unroll
+      for (int p = 1; p < PARTS; ++p) FR_ISSUE_PART(k_tiles - 1, sp, p);
+    }
     for (; kt < k_tiles - 1; ++kt) {
-      const int xn = (xs + 1 == SX) ? 0 : xs + 1, wn = (ws + 1 == SW) ? 0 : ws + 1;
+      const int sn = (sl + 1 == S) ? 0 : sl + 1;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         if (ks + 1 < KS) {
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(xs, ws, ks + 1, (ks + 1) & 1));
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), {});
         } else {
           asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
           __builtin_amdgcn_s_barrier();
-          if (kt + SX < k_tiles) FR_ISSUE_X(kt + SX, xs);
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(xn, wn, 0, 0));
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, sn, 0, 0), {});
         }
       }
-      xs = xn;
-      ws = wn;
+      sl = sn;
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {  // last tile
       if (ks + 1 < KS) {
-        FR_KSTEP(ks & 1, FR_READ_FRAGS(xs, ws, ks + 1, (ks + 1) & 1));
+        FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), {});
       } else {
-        FR_KSTEP(ks & 1, {});
+        FR_KSTEP(ks & 1, {}, {});
       }
     }
 #undef FR_KSTEP
-#undef FR_ISSUE_X
-#undef FR_ISSUE_W
+#undef FR_ISSUE_PART
   }
 #undef FR_READ_FRAGS
 #undef FR_MMA
