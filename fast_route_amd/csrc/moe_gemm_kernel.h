@@ -330,62 +330,83 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
 #undef FR_COMPUTE_TILE
   } else {
     // ---- direct-to-LDS ring --------------------------------------------------
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer resources and LDS-DMA builtins exist in the device pass only
     // A wavefront-wide global_load_lds_dwordx4 fills 64 consecutive 16-byte LDS
     // slots (slot = row*CPR + physical chunk), lane L the L-th of them, so each
     // lane fetches the logical chunk that the swizzle maps to its slot.
-    typedef const __attribute__((address_space(1))) void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
     constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, NL = XI + WI;
-    // The NL loads that refill a slot are issued in PARTS groups of PER, one group per
-    // K-step, so the data does not arrive at the LDS in one burst that starves ds_read.
-    constexpr int PARTS = C::SPREAD < 1 ? 1 : (C::SPREAD > KS - 1 ? (KS > 1 ? KS - 1 : 1) : C::SPREAD);
+    // The NL loads that refill a slot are issued in PARTS groups of PER, one group per K-step.
+    constexpr int PARTS = C::SPREAD < 1 ? 1 : (C::SPREAD > KS ? KS : C::SPREAD);
     constexpr int PER = (NL + PARTS - 1) / PARTS, P0 = PER < NL ? PER : NL;
     static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
     static_assert((S - 1) * NL <= 63, "vmcnt budget");
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const T* xsrc[XI];
-    const T* wsrc[WI];
+    // Loads are buffer-addressed: a scalar resource (base of X, base of this expert's
+    // W), one 32-bit byte offset per lane and the K offset of the tile as the scalar
+    // offset.  Per-lane 64-bit addresses cost two VALU adds per load and twice the
+    // address traffic to the texture unit, and a wavefront that issues a burst of them
+    // sits in the issue stage (no MFMAs) until the unit has taken them all.
+    // Offsets are 32-bit: slot-addressed token rows are taken relative to the tile's
+    // first row; gathered rows and an expert's weights must span less than 4 GiB
+    // (checked by the launcher).
+    const int64_t xrow0 = a.top_k > 0 ? 0 : static_cast<int64_t>(pid_t) * BT;
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(X + xrow0 * a.ldx), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(W), 0, -1, 0x00020000);
+    unsigned xsrc[XI], wsrc[WI];  // byte offsets
 #pragma unroll
     for (int i = 0; i < XI; ++i) {
       const int slot = (i * NW + wave_u) * kWave + lane;
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
-      xsrc[i] = X + x_src_row(rr) * a.ldx + k0 + c * EPC;
+      xsrc[i] = static_cast<unsigned>(((x_src_row(rr) - xrow0) * a.ldx + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));
     }
 #pragma unroll
     for (int i = 0; i < WI; ++i) {
       const int slot = (i * NW + wave_u) * kWave + lane;
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
-      wsrc[i] = W + static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * EPC;
+      wsrc[i] = static_cast<unsigned>((static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));
     }
-    // group p_ of the loads of tile tile_ into ring slot slot_: token-tile loads first
-#define FR_ISSUE_PART(tile_, slot_, p_)                                                                    \
+    // load q_ (token-tile loads first, then weight-tile loads) of tile tile_ into ring slot slot_
+#define FR_ISSUE_ONE(tile_, slot_, q_)                                                                     \
   {                                                                                                        \
-    _Pragma("unroll") for (int q = (p_) * PER; q < ((p_) + 1) * PER && q < NL; ++q) {                      \
-      if (q < XI) {                                                                                        \
-        __builtin_amdgcn_global_load_lds(                                                                  \
-            (gptr_t)(xsrc[q < XI ? q : 0] + (tile_) * BK),                                                 \
-            (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + (q * NW + wave_u) * (kWave * 16)), 16, 0, 0);     \
-      } else {                                                                                             \
-        __builtin_amdgcn_global_load_lds(                                                                  \
-            (gptr_t)(wsrc[q < XI ? 0 : q - XI] + (tile_) * BK),                                            \
-            (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + ((q - XI) * NW + wave_u) * (kWave * 16)), \
-            16, 0, 0);                                                                                     \
-      }                                                                                                    \
+    if ((q_) < XI) {                                                                                       \
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
+          xrs, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((q_) * NW + wave_u) * (kWave * 16)), 16,      \
+          xsrc[(q_) < XI ? (q_) : 0], (tile_) * C::BKB, 0, 0);                                             \
+    } else {                                                                                               \
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
+          wrs, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) - XI) * NW + wave_u) * (kWave * 16)), \
+          16, wsrc[(q_) < XI ? 0 : (q_) - XI], (tile_) * C::BKB, 0, 0);                                    \
     }                                                                                                      \
   }
-    // One K-step: the first half of the MFMAs covers the LDS latency of the fragments
-    // of the NEXT step, which are read into the other fragment buffer; a group of
-    // refill loads, if any, goes out between the halves.
-    constexpr int JSPLIT = (C::JF + 1) / 2;
-#define FR_KSTEP(fb_, READ_NEXT, ISSUE)          \
-  {                                              \
-    FR_MMA(fb_, 0, JSPLIT);                      \
-    __builtin_amdgcn_sched_barrier(0);           \
-    READ_NEXT;                                   \
-    ISSUE;                                       \
-    __builtin_amdgcn_sched_barrier(0);           \
-    FR_MMA(fb_, JSPLIT, C::JF);                  \
-    __builtin_amdgcn_sched_barrier(0);           \
+#define FR_ISSUE_PART(tile_, slot_, p_)                                                                    \
+  {                                                                                                        \
+    _Pragma("unroll") for (int q = (p_) * PER; q < ((p_) + 1) * PER && q < NL; ++q) FR_ISSUE_ONE(tile_, slot_, q); \
+  }
+    // One K-step: NM MFMAs.  The fragments of the NEXT step are read into the other
+    // fragment buffer after the first half, so the second half covers the LDS latency.
+    // The refill loads of group p_ (if HAVE_) go out one at a time, evenly spaced
+    // between the MFMAs.
+    constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
+#define FR_KSTEP(fb_, READ_NEXT, HAVE_, tile_, slot_, p_)                                     \
+  {                                                                                           \
+    _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                          \
+      const int j = m / C::IT, i = m % C::IT;                                                 \
+      if constexpr (C::TILE == 32) acc[j][i] = E::m32(wfr[fb_][j], xf[fb_][i], acc[j][i]);    \
+      else acc[j][i] = E::m16(wfr[fb_][j], xf[fb_][i], acc[j][i]);                            \
+      __builtin_amdgcn_sched_barrier(0);                                                      \
+      if (m == RD_AT) {                                                                       \
+        READ_NEXT;                                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                    \
+      }                                                                                       \
+      if (HAVE_) {                                                                            \
+        _Pragma("unroll") for (int r = 0; r < PER; ++r)                                       \
+          if (m == ((2 * r + 1) * NM) / (2 * PER) && (p_) * PER + r < NL) {                   \
+            FR_ISSUE_ONE(tile_, slot_, (p_) * PER + r);                                       \
+            __builtin_amdgcn_sched_barrier(0);                                                \
+          }                                                                                   \
+      }                                                                                       \
+    }                                                                                         \
   }
     // Software pipeline.  Tiles are loaded in order; the barrier that publishes tile
     // kt+1 sits before the LAST K-step of tile kt (whose fragments are already in
@@ -417,13 +438,12 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         if (ks + 1 < KS) {
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1),
-                   if (ks + 1 < PARTS) FR_ISSUE_PART(kt - 1 + S, sp, ks + 1));
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), ks + 1 < PARTS, kt - 1 + S, sp, ks + 1);
         } else {
           // tile kt+1 landed (this lane's part) and this wavefront's reads of tile kt are done
           asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((S - 2) * NL) : "memory");
           __builtin_amdgcn_s_barrier();  // ... everyone's: the slot of tile kt can be refilled
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, sn, 0, 0), FR_ISSUE_PART(kt + S, sl, 0));
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, sn, 0, 0), true, kt + S, sl, 0);
         }
       }
       sl = sn;
@@ -439,11 +459,11 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         if (ks + 1 < KS) {
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), {});
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), false, 0, 0, 0);
         } else {
           asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
           __builtin_amdgcn_s_barrier();
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, sn, 0, 0), {});
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, sn, 0, 0), false, 0, 0, 0);
         }
       }
       sl = sn;
@@ -451,13 +471,15 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {  // last tile
       if (ks + 1 < KS) {
-        FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), {});
+        FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), false, 0, 0, 0);
       } else {
-        FR_KSTEP(ks & 1, {}, {});
+        FR_KSTEP(ks & 1, {}, false, 0, 0, 0);
       }
     }
 #undef FR_KSTEP
 #undef FR_ISSUE_PART
+#undef FR_ISSUE_ONE
+#endif
   }
 #undef FR_READ_FRAGS
 #undef FR_MMA
@@ -549,6 +571,14 @@ int launch_gemm(const GemmArgs& a, int splits, hipStream_t st) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
     if (e != hipSuccess) return fail(FR_E_LAUNCH, "hipFuncSetAttribute(%d B LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
     attr_set = true;
+  }
+  if (C::STAGES > 0) {  // the ring loads address rows by 32-bit byte offsets
+    const int64_t x_rows = a.top_k > 0 ? a.num_valid / a.top_k : C::BT;
+    const int64_t w_rows = EPI == EPI_SILU ? 2 * static_cast<int64_t>(a.N) : a.N;
+    const int64_t lim = int64_t(1) << 32, es = sizeof(T);
+    if (x_rows * a.ldx * es >= lim || w_rows * a.ldw * es >= lim)
+      return fail(FR_E_SHAPE, "token rows (%lld x %lld) or one expert's weights (%lld x %lld) span 4 GiB or more",
+                  (long long)x_rows, (long long)a.ldx, (long long)w_rows, (long long)a.ldw);
   }
   const unsigned grid_x = static_cast<unsigned>(a.num_t_blocks) * static_cast<unsigned>(a.num_f_tiles);
   hipLaunchKernelGGL((moe_gemm_kernel<T, C, EPI>), dim3(grid_x, splits), dim3(C::NT), C::LDS_BYTES, st, a);
