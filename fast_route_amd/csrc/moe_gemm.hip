@@ -31,13 +31,17 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
 //   64 rows:        8 wavefronts, register-staged double buffer (op-level API only;
 //                   the fused layer goes from 32-row to 128-row blocks);
 //   32 / 16 rows:   decode regime, 16x16 MFMA, 3-slot ring, two workgroups per CU:
-//                   weight streaming at HBM rate.
+//                   weight streaming at HBM rate.  The gate/up GEMM (short weight rows
+//                   of H elements, many of them) streams faster with 512-byte row
+//                   segments: T32L / T16L, used when H allows.
 template <typename T> struct Tiles {  // bf16 / fp16
   typedef Cfg<256, 256, 128, 4, 2, 32, 1, 2> T256;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
   typedef Cfg<32, 128, 128, 1, 4, 16, 2, 3> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
+  typedef Cfg<32, 128, 512, 1, 4, 16, 1, 2> T32L;
+  typedef Cfg<16, 128, 512, 1, 4, 16, 1, 2> T16L;
 };
 template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per two K-steps
   typedef Cfg<256, 256, 128, 4, 2, 32, 1, 2> T256;
@@ -45,6 +49,8 @@ template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
   typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
+  typedef Cfg<32, 128, 512, 1, 4, 16, 1, 2> T32L;
+  typedef Cfg<16, 128, 512, 1, 4, 16, 1, 2> T16L;
 };
 
 bool valid_block(int block) { return block == 16 || block == 32 || block == 64 || block == 128 || block == 256; }
@@ -67,8 +73,20 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
     case 256: fill(256, TL::T256::BF, TL::T256::BKB); return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
     case 128: fill(128, TL::T128::BF, TL::T128::BKB); return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
     case 64: fill(64, TL::T64::BF, TL::T64::BKB); return launch_gemm<T, typename TL::T64, EPI>(a, splits, st);
-    case 32: fill(32, TL::T32::BF, TL::T32::BKB); return launch_gemm<T, typename TL::T32, EPI>(a, splits, st);
-    case 16: fill(16, TL::T16::BF, TL::T16::BKB); return launch_gemm<T, typename TL::T16, EPI>(a, splits, st);
+    case 32:
+      if (EPI == EPI_SILU && a.K % (TL::T32L::BKB / static_cast<int>(sizeof(T))) == 0) {
+        fill(32, TL::T32L::BF, TL::T32L::BKB);
+        return launch_gemm<T, typename TL::T32L, EPI>(a, splits, st);
+      }
+      fill(32, TL::T32::BF, TL::T32::BKB);
+      return launch_gemm<T, typename TL::T32, EPI>(a, splits, st);
+    case 16:
+      if (EPI == EPI_SILU && a.K % (TL::T16L::BKB / static_cast<int>(sizeof(T))) == 0) {
+        fill(16, TL::T16L::BF, TL::T16L::BKB);
+        return launch_gemm<T, typename TL::T16L, EPI>(a, splits, st);
+      }
+      fill(16, TL::T16::BF, TL::T16::BKB);
+      return launch_gemm<T, typename TL::T16, EPI>(a, splits, st);
     default: return fail(FR_E_SHAPE, "routing block %d not in {16, 32, 64, 128, 256}", block);
   }
 }
