@@ -199,6 +199,19 @@ def kernel_roofline(shape, rec, fp8=False):
             "avg_launch_us": round(dur * 1e6, 2), "algorithmic_bytes_per_launch": byts}
 
 
+def recorded_traffic(metric):
+    """HBM bytes per launch of the dominant kernel for this workload, as measured offline with
+    rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE runs, scaled by the copy probe) and recorded
+    in profiles/hbm_traffic.json; None when the workload has no record."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            rec = json.load(f).get(metric)
+    except (OSError, ValueError):
+        return None
+    return rec["traffic_bytes"] if rec else None
+
+
 def cpu_baseline(torch, shape, layer, sample_tokens):
     """fp32 PyTorch oracle on the host cores over the first `sample_tokens` tokens of the same batch."""
     import oracle
@@ -282,6 +295,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=1024)
     ap.add_argument("--routing", action="store_true", help="also time the routing-only stress workload")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 1 GiB device copy: the kernel of known size that calibrates "
+                         "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X runs the whole layer); --gpus must be 1")
@@ -326,6 +342,14 @@ def main():
         "roofline": kernel_roofline(shape, head, fp8 is not None),
         "sweep": sweep,
     }
+    result["roofline"]["traffic"] = recorded_traffic(result["metric"])
+    if args.copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)  # an elementwise kernel (copy_ would take the DMA engine)
+        torch.cuda.synchronize()
+        result["copy_probe"] = {"kernel": "torch.mul(src, 1.0, out=dst), fp32", "bytes_read": src.numel() * 4, "bytes_written": dst.numel() * 4, "launches": 3}
     if args.routing:
         result["routing_stress"] = routing_bench(torch, N, args.steps, args.warmup, args.seed)
     if not args.no_cpu and fp8 is None:
