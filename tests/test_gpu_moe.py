@@ -99,6 +99,33 @@ def test_layer_edge_cases(native):
     _assert_close(out, oracle.moe_experts(x, w1, w2, w.half().float(), ids), dtype, "dtype coercion")
 
 
+@pytest.mark.parametrize("M", [4, 40])
+def test_hidden_size_not_multiple_of_long_row_tile(native, M):
+    """H = 384 is a multiple of 128 but not of 256: the decode gate/up GEMM must take the
+    short-row tile instead of the 512-byte-row one."""
+    from fast_route_amd import fused_moe
+    _say(f"layer H=384 M={M}")
+    x, logits, w1, w2 = _inputs(M, 384, 256, 8, 5, torch.bfloat16)
+    out = fused_moe(x.cuda(), w1.cuda(), w2.cuda(), logits.cuda(), 2, True)
+    torch.cuda.synchronize()
+    _assert_close(out, oracle.fused_moe(x, w1, w2, logits, 2, True), torch.bfloat16, f"H=384 M={M}")
+
+
+def test_token_matrix_of_4gib_is_refused(native):
+    """Tile loads address rows by 32-bit byte offsets: a gathered token matrix of 4 GiB
+    or more is refused before anything is launched (no memory of that size is touched)."""
+    from fast_route_amd import _native as N
+    H, Fd, E, k, block = 256, 128, 2, 1, 16
+    M = (1 << 32) // (H * 2)  # M*H*2 bytes == 4 GiB exactly
+    dummy = torch.zeros(1 << 16, dtype=torch.int32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    rc = N.lib().fr_moe_gateup_silu(dummy.data_ptr(), dummy.data_ptr(), dummy.data_ptr(), dummy.data_ptr(),
+                                    dummy.data_ptr(), M, H, Fd, E, k, block, N.FR_BF16, dummy.data_ptr(), st)
+    assert rc == -2, rc
+    assert b"4 GiB" in N.lib().fr_last_error_string()
+    torch.cuda.synchronize()
+
+
 def test_layer_rejects_bad_arguments(native):
     from fast_route_amd import fused_moe
     x, logits, w1, w2 = _inputs(8, 256, 128, 8, 3, torch.bfloat16)
