@@ -28,6 +28,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
 // Token-block sizes and their tile shapes.  K tiles are 128 bytes per row (256 for
 // the 16-row block); every block except 64 streams tiles HBM -> LDS directly.
 //   256 / 128 rows: 8 wavefronts, 32x32 MFMA, 2- or 3-slot ring (compute-bound regime);
+//                   in the 256-row tile one wavefront per SIMD issues the loads of both;
 //   64 rows:        8 wavefronts, register-staged double buffer (op-level API only;
 //                   the fused layer goes from 32-row to 128-row blocks);
 //   32 / 16 rows:   decode regime, 16x16 MFMA, 3-slot ring, two workgroups per CU:
@@ -35,7 +36,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
 //                   of H elements, many of them) streams faster with 512-byte row
 //                   segments: T32L / T16L, used when H allows.
 template <typename T> struct Tiles {  // bf16 / fp16
-  typedef Cfg<256, 256, 128, 4, 2, 32, 1, 2> T256;
+  typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
   typedef Cfg<32, 128, 128, 1, 4, 16, 2, 3> T32;
@@ -44,7 +45,7 @@ template <typename T> struct Tiles {  // bf16 / fp16
   typedef Cfg<16, 128, 512, 1, 4, 16, 1, 2> T16L;
 };
 template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per two K-steps
-  typedef Cfg<256, 256, 128, 4, 2, 32, 1, 2> T256;
+  typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
   typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;

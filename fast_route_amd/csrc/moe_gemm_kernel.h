@@ -106,10 +106,11 @@ __device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); 
 // flight).  STAGES >= 2: tiles go HBM -> LDS directly (global_load_lds_dwordx4)
 // through rings of STAGES token-tile and weight-tile slots; a slot is refilled once
 // its tile's last fragments are in registers, the loads spread over SPREAD K-steps.
-template <int BT_, int BF_, int BKB_, int WT_, int WF_, int TILE_, int MINB_ = 1, int STAGES_ = 0, int SPREAD_ = 0>
+template <int BT_, int BF_, int BKB_, int WT_, int WF_, int TILE_, int MINB_ = 1, int STAGES_ = 0, int SPREAD_ = 0, int IW_ = 1>
 struct Cfg {
   static constexpr int BT = BT_, BF = BF_, BKB = BKB_, WT = WT_, WF = WF_, TILE = TILE_, MINB = MINB_;
   static constexpr int STAGES = STAGES_;  // ring slots of the token and of the weight tiles
+  static constexpr int IW = IW_;          // 2: only the first half of the wavefronts issue tile loads, each for two
   static constexpr int SPREAD = SPREAD_;  // K-steps over which the refill of a slot is spread (<= 1: one burst)
   static constexpr int NBUF = STAGES_ == 0 ? 2 : STAGES_;
   static constexpr int NT = WT * WF * kWave;       // threads
@@ -338,9 +339,13 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, NL = XI + WI;
     // The NL loads that refill a slot are issued in PARTS groups of PER, one group per K-step.
     constexpr int PARTS = C::SPREAD < 1 ? 1 : (C::SPREAD > KS ? KS : C::SPREAD);
-    constexpr int PER = (NL + PARTS - 1) / PARTS, P0 = PER < NL ? PER : NL;
+    // With IW == 2 the loads of wavefront w + NW/2 are issued by wavefront w: the two share a SIMD, so while
+    // one sits in the load issue stage the other keeps the MFMA pipe busy instead of both stalling together.
+    constexpr int IW = C::IW, NLI = NL * IW;  // loads per issuing wavefront per tile
+    constexpr int PER = (NLI + PARTS - 1) / PARTS, P0 = PER < NLI ? PER : NLI;
+    static_assert(IW >= 1 && NW % IW == 0, "issue width");
     static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
-    static_assert((S - 1) * NL <= 63, "vmcnt budget");
+    static_assert((S - 1) * NLI <= 63, "vmcnt budget");
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     // Loads are buffer-addressed: a scalar resource (base of X, base of this expert's
     // W), one 32-bit byte offset per lane and the K offset of the tile as the scalar
@@ -353,35 +358,40 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     const int64_t xrow0 = a.top_k > 0 ? 0 : static_cast<int64_t>(pid_t) * BT;
     const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(X + xrow0 * a.ldx), 0, -1, 0x00020000);
     const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(W), 0, -1, 0x00020000);
-    unsigned xsrc[XI], wsrc[WI];  // byte offsets
+    const bool issuer = wave_u < NW / IW;
+    unsigned xsrc[XI * IW], wsrc[WI * IW];  // byte offsets, [load][virtual wavefront]
 #pragma unroll
-    for (int i = 0; i < XI; ++i) {
-      const int slot = (i * NW + wave_u) * kWave + lane;
+    for (int ih = 0; ih < XI * IW; ++ih) {
+      const int i = ih / IW, vw = (wave_u + (ih % IW) * (NW / IW)) % NW;
+      const int slot = (i * NW + vw) * kWave + lane;
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
-      xsrc[i] = static_cast<unsigned>(((x_src_row(rr) - xrow0) * a.ldx + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));
+      xsrc[ih] = static_cast<unsigned>(((x_src_row(rr) - xrow0) * a.ldx + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));
     }
 #pragma unroll
-    for (int i = 0; i < WI; ++i) {
-      const int slot = (i * NW + wave_u) * kWave + lane;
+    for (int ih = 0; ih < WI * IW; ++ih) {
+      const int i = ih / IW, vw = (wave_u + (ih % IW) * (NW / IW)) % NW;
+      const int slot = (i * NW + vw) * kWave + lane;
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
-      wsrc[i] = static_cast<unsigned>((static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));
+      wsrc[ih] = static_cast<unsigned>((static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));
     }
-    // load q_ (token-tile loads first, then weight-tile loads) of tile tile_ into ring slot slot_
+    // load q_ of an issuing wavefront (token-tile loads first, then weight-tile loads; the IW
+    // virtual wavefronts of one load index are adjacent) of tile tile_ into ring slot slot_
 #define FR_ISSUE_ONE(tile_, slot_, q_)                                                                     \
   {                                                                                                        \
-    if ((q_) < XI) {                                                                                       \
+    const int vw_ = wave_u + ((q_) % IW) * (NW / IW);                                                      \
+    if ((q_) < XI * IW) {                                                                                  \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
-          xrs, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((q_) * NW + wave_u) * (kWave * 16)), 16,      \
-          xsrc[(q_) < XI ? (q_) : 0], (tile_) * C::BKB, 0, 0);                                             \
+          xrs, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + (((q_) / IW) * NW + vw_) * (kWave * 16)), 16,  \
+          xsrc[(q_) < XI * IW ? (q_) : 0], (tile_) * C::BKB, 0, 0);                                        \
     } else {                                                                                               \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
-          wrs, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) - XI) * NW + wave_u) * (kWave * 16)), \
-          16, wsrc[(q_) < XI ? 0 : (q_) - XI], (tile_) * C::BKB, 0, 0);                                    \
+          wrs, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + ((((q_) - XI * IW) / IW) * NW + vw_) * (kWave * 16)), \
+          16, wsrc[(q_) < XI * IW ? 0 : (q_) - XI * IW], (tile_) * C::BKB, 0, 0);                          \
     }                                                                                                      \
   }
 #define FR_ISSUE_PART(tile_, slot_, p_)                                                                    \
   {                                                                                                        \
-    _Pragma("unroll") for (int q = (p_) * PER; q < ((p_) + 1) * PER && q < NL; ++q) FR_ISSUE_ONE(tile_, slot_, q); \
+    _Pragma("unroll") for (int q = (p_) * PER; q < ((p_) + 1) * PER && q < NLI; ++q) FR_ISSUE_ONE(tile_, slot_, q); \
   }
     // One K-step: NM MFMAs.  The fragments of the NEXT step are read into the other
     // fragment buffer after the first half, so the second half covers the LDS latency.
@@ -401,7 +411,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
       }                                                                                       \
       if (HAVE_) {                                                                            \
         _Pragma("unroll") for (int r = 0; r < PER; ++r)                                       \
-          if (m == ((2 * r + 1) * NM) / (2 * PER) && (p_) * PER + r < NL) {                   \
+          if (m == ((2 * r + 1) * NM) / (2 * PER) && (p_) * PER + r < NLI) {                   \
             FR_ISSUE_ONE(tile_, slot_, (p_) * PER + r);                                       \
             __builtin_amdgcn_sched_barrier(0);                                                \
           }                                                                                   \
@@ -413,69 +423,73 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     // registers).  After it the slot of tile kt is refilled with tile kt+S: group 0 in
     // that last K-step, groups 1.. in the first K-steps of tile kt+1.  vmcnt counts
     // loads in issue order, so "tile kt+1 landed" leaves exactly the S-2 later tiles
-    // outstanding.  The prologue leaves tile S-1 in the same half-issued state.
-#pragma unroll
-    for (int t = 0; t < S; ++t) {
-      if (t < k_tiles) {
-        FR_ISSUE_PART(t, t, 0);
-        if (t < S - 1) {
-#pragma unroll
-          for (int p = 1; p < PARTS; ++p) FR_ISSUE_PART(t, t, p);
-        }
-      }
-    }
-    if (k_tiles >= S) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((S - 2) * NL + P0) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    FR_READ_FRAGS(0, 0, 0, 0);
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): no scalar load may be pending when the loop starts
-    int sl = 0;  // ring slot of tile kt
-    // steady state: tile kt+S exists, so the body is one basic block with a fixed vmcnt
-    // and the compiler can count the outstanding LDS reads exactly
-    int kt = 0;
-    for (; kt < k_tiles - S; ++kt) {
-      const int sn = (sl + 1 == S) ? 0 : sl + 1, sp = (sl == 0) ? S - 1 : sl - 1;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        if (ks + 1 < KS) {
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), ks + 1 < PARTS, kt - 1 + S, sp, ks + 1);
-        } else {
-          // tile kt+1 landed (this lane's part) and this wavefront's reads of tile kt are done
-          asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((S - 2) * NL) : "memory");
-          __builtin_amdgcn_s_barrier();  // ... everyone's: the slot of tile kt can be refilled
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, sn, 0, 0), true, kt + S, sl, 0);
-        }
-      }
-      sl = sn;
-    }
-    // drain: finish the half-issued refill (the last tile), then no more loads
-    if (k_tiles >= S) {
-      const int sp = (sl == 0) ? S - 1 : sl - 1;
-#pragma unroll
-      for (int p = 1; p < PARTS; ++p) FR_ISSUE_PART(k_tiles - 1, sp, p);
-    }
-    for (; kt < k_tiles - 1; ++kt) {
-      const int sn = (sl + 1 == S) ? 0 : sl + 1;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        if (ks + 1 < KS) {
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), false, 0, 0, 0);
-        } else {
-          asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-          __builtin_amdgcn_s_barrier();
-          FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, sn, 0, 0), false, 0, 0, 0);
-        }
-      }
-      sl = sn;
-    }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {  // last tile
-      if (ks + 1 < KS) {
-        FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), false, 0, 0, 0);
-      } else {
-        FR_KSTEP(ks & 1, {}, false, 0, 0, 0);
-      }
-    }
+    // outstanding.  The prologue leaves tile S-1 in the same half-issued state.  Inside the
+    // steady loop tile kt+S exists, so its body is one basic block with a fixed vmcnt and the
+    // compiler counts the outstanding LDS reads exactly; the drain finishes the half-issued
+    // refill of the last tile and issues nothing more.  ISS_: this wavefront issues loads.
+#define FR_PIPELINE(ISS_) \
+  { \
+_Pragma("unroll") \
+    for (int t = 0; t < S; ++t) { \
+      if (t < k_tiles) { \
+        if (ISS_) FR_ISSUE_PART(t, t, 0); \
+        if (t < S - 1) { \
+_Pragma("unroll") \
+          for (int p = 1; p < PARTS; ++p) if (ISS_) FR_ISSUE_PART(t, t, p); \
+        } \
+      } \
+    } \
+    if (k_tiles >= S) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((S - 2) * NLI + P0) : "memory"); \
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); \
+    __builtin_amdgcn_s_barrier(); \
+    FR_READ_FRAGS(0, 0, 0, 0); \
+    __builtin_amdgcn_s_waitcnt(0xC07F); \
+    int sl = 0; \
+    int kt = 0; \
+    for (; kt < k_tiles - S; ++kt) { \
+      const int sn = (sl + 1 == S) ? 0 : sl + 1, sp = (sl == 0) ? S - 1 : sl - 1; \
+_Pragma("unroll") \
+      for (int ks = 0; ks < KS; ++ks) { \
+        if (ks + 1 < KS) { \
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), (ISS_) && ks + 1 < PARTS, kt - 1 + S, sp, ks + 1); \
+        } else { \
+          asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((S - 2) * NLI) : "memory"); \
+          __builtin_amdgcn_s_barrier(); \
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, sn, 0, 0), ISS_, kt + S, sl, 0); \
+        } \
+      } \
+      sl = sn; \
+    } \
+    if (k_tiles >= S) { \
+      const int sp = (sl == 0) ? S - 1 : sl - 1; \
+_Pragma("unroll") \
+      for (int p = 1; p < PARTS; ++p) if (ISS_) FR_ISSUE_PART(k_tiles - 1, sp, p); \
+    } \
+    for (; kt < k_tiles - 1; ++kt) { \
+      const int sn = (sl + 1 == S) ? 0 : sl + 1; \
+_Pragma("unroll") \
+      for (int ks = 0; ks < KS; ++ks) { \
+        if (ks + 1 < KS) { \
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), false, 0, 0, 0); \
+        } else { \
+          asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); \
+          __builtin_amdgcn_s_barrier(); \
+          FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, sn, 0, 0), false, 0, 0, 0); \
+        } \
+      } \
+      sl = sn; \
+    } \
+_Pragma("unroll") \
+    for (int ks = 0; ks < KS; ++ks) { \
+      if (ks + 1 < KS) { \
+        FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, sl, ks + 1, (ks + 1) & 1), false, 0, 0, 0); \
+      } else { \
+        FR_KSTEP(ks & 1, {}, false, 0, 0, 0); \
+      } \
+    } \
+  }
+    if (IW == 1 || issuer) FR_PIPELINE(true) else FR_PIPELINE(false)
+#undef FR_PIPELINE
 #undef FR_KSTEP
 #undef FR_ISSUE_PART
 #undef FR_ISSUE_ONE
