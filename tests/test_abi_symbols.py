@@ -64,11 +64,13 @@ def test_reference_import_paths_resolve():
     """The reference's module paths (SURVEY: fast_route.layers.*, fast_route.ops.*) import here."""
     from fast_route.layers.stable_route import fused_moe as a
     from fast_route.layers.vllm_route import fused_moe as b
+    from fast_route.layers.profile_fused_route import fused_moe as c
     from fast_route.ops.stable_route import fused_route
     from fast_route.ops.fused_moe import invoke_fused_moe_kernel, moe_align_block_size
     import inspect
     assert list(inspect.signature(a).parameters) == ["hidden_states", "gate", "w1", "w2", "topk", "renormalize", "inplace"]
     assert list(inspect.signature(b).parameters) == ["hidden_states", "gate", "w1", "w2", "topk", "renormalize", "inplace"]
+    assert list(inspect.signature(c).parameters)[:7] == ["hidden_states", "gate", "w1", "w2", "topk", "renormalize", "inplace"]
     assert list(inspect.signature(fused_route).parameters) == ["hidden_state", "gate", "topk", "topk_weights", "topk_ids", "renormalize"]
     assert list(inspect.signature(moe_align_block_size).parameters) == ["topk_ids", "block_size", "num_experts"]
     assert list(inspect.signature(invoke_fused_moe_kernel).parameters)[:4] == ["A", "B", "C", "topk_weights"]

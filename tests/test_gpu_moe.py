@@ -190,6 +190,47 @@ def test_stable_and_vllm_route_layers(native):
     _assert_close(b, refb, dtype, "vllm_route layer")
 
 
+def test_profile_twin_matches_layer_and_writes_trace(native, tmp_path):
+    """layers/profile_fused_route.py: same result as the fused layer, bit for bit (same
+    kernels, same plan), and a chrome trace with one complete event per stage."""
+    import json
+    from fast_route_amd.layers import profile_fused_route, stable_route
+    _say("profile twin")
+    dtype = torch.bfloat16
+    M, H, Fd, E, k = 96, 512, 256, 8, 2
+    x, _, w1, w2 = _inputs(M, H, Fd, E, 12, dtype)
+    gate = (torch.randn(H, E, generator=torch.Generator().manual_seed(2)) / 8).to(dtype)
+    ref = stable_route.fused_moe(x.cuda(), gate.cuda(), w1.cuda(), w2.cuda(), k, True)
+    out = profile_fused_route.fused_moe(x.cuda(), gate.cuda(), w1.cuda(), w2.cuda(), k, True, save_dir=str(tmp_path))
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+    path = tmp_path / f"fused_breakdown_{M}_{H}_{E}_{2 * Fd}_{k}.json"
+    trace = json.loads(path.read_text())
+    names = [e["name"] for e in trace["traceEvents"]]
+    assert names == list(profile_fused_route.STAGES)
+    assert all(e["ph"] == "X" and e["dur"] > 0 for e in trace["traceEvents"])
+    ts = [e["ts"] for e in trace["traceEvents"]]
+    assert ts == sorted(ts)
+
+
+def test_transformer_layer_bench_runs_and_matches_its_parts(native):
+    """fast_route_amd.transformer_layer_bench: the layer is attention + residual + the
+    gate-matrix MoE; its output equals the MoE entry point applied to attn(x) + x."""
+    from fast_route_amd import transformer_layer_bench as tb
+    from fast_route_amd.layers.stable_route import fused_moe
+    _say("transformer layer bench")
+    rec, out, (gate, w1, w2, attn) = tb.run(seq=64, n=256, k=512, e=8, topk=2, b=2, n_head=4, head_dim=64,
+                                            reps=3, warmup=1)
+    assert out.shape == (2 * 64, 512) and torch.isfinite(out.float()).all()
+    assert 0.0 < rec["moe_share"] <= 1.0 and rec["layer_ms"] > 0 and rec["layer_ms_p20"] <= rec["layer_ms_p80"]
+    g = torch.Generator(device="cuda").manual_seed(1337)
+    x = torch.randn((2, 64, 512), device="cuda", dtype=torch.float16, generator=g) / 10
+    with torch.no_grad():
+        h = (attn(x) + x).view(-1, 512)
+        again = fused_moe(h, gate, w1, w2, 2, True, False)
+    assert torch.equal(out, again)
+
+
 def test_mixtral_shape_sampled_tokens_and_properties(native):
     """BASELINE config 2 at full size (H4096 F14336 E8 top2): oracle on a sample of
     tokens, plus size-independent properties on all of them."""
