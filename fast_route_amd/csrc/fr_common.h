@@ -17,6 +17,11 @@ int check_launch(const char* what);
 int quant_rows(const void* x, int dtype, int64_t rows, const int32_t* rows_dev, int64_t K, int64_t ldx, void* q_out,
                float* scale_out, hipStream_t st);
 
+// gating + routing arrays in one launch (small batches); see routing.hip
+bool route_align_fits(int64_t M, int E, int topk);
+int route_align_small(const void* logits, int logits_dtype, int64_t M, int E, int topk, int renorm, int block,
+                      float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, hipStream_t st);
+
 #define FR_REQUIRE(cond, code, ...) \
   do {                              \
     if (!(cond)) return ::fr::fail((code), __VA_ARGS__); \

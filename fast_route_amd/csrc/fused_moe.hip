@@ -110,6 +110,22 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   return FR_OK;
 }
 
+namespace fr {
+namespace {
+// top-k gating of the logits and the routing arrays of the result: one launch for small
+// batches, gating then align otherwise
+int route_and_align(const void* logits, int logits_dtype, int64_t M, int E, int topk, int renormalize, int block,
+                    const Carve& c, void* stream) {
+  if (route_align_fits(M, E, topk))
+    return route_align_small(logits, logits_dtype, M, E, topk, renormalize, block, c.topk_w, c.topk_ids, c.sorted,
+                             c.expert_ids, c.npost, static_cast<hipStream_t>(stream));
+  int rc = fr_gating_topk(logits, logits_dtype, M, E, E, topk, renormalize, c.topk_w, c.topk_ids, stream);
+  if (rc != FR_OK) return rc;
+  return fr_moe_align(c.topk_ids, FR_I32, M * topk, E, block, c.sorted, c.expert_ids, c.npost, c.align_ws, c.align_ws_bytes, stream);
+}
+}  // namespace
+}  // namespace fr
+
 extern "C" int fr_fused_experts(const void* x, const void* w1, const void* w2, const float* topk_weights,
                                 const int32_t* topk_ids, int64_t M, int64_t H, int64_t F, int E, int topk,
                                 int dtype, void* out, void* workspace, int64_t workspace_bytes, void* stream) {
@@ -139,9 +155,11 @@ extern "C" int fr_fused_moe(const void* x, const void* w1, const void* w2, const
   FR_REQUIRE(workspace && workspace_bytes >= p.workspace_bytes, FR_E_WORKSPACE, "fr_fused_moe: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)p.workspace_bytes);
   FR_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FR_E_ALIGN, "fr_fused_moe: workspace must be 256-byte aligned");
   Carve c = carve(workspace, M, H, F, E, topk, dtype, p);
-  rc = fr_gating_topk(logits, logits_dtype, M, E, E, topk, renormalize, c.topk_w, c.topk_ids, stream);
+  rc = route_and_align(logits, logits_dtype, M, E, topk, renormalize, p.block, c, stream);
   if (rc != FR_OK) return rc;
-  return fr_fused_experts(x, w1, w2, c.topk_w, c.topk_ids, M, H, F, E, topk, dtype, out, workspace, workspace_bytes, stream);
+  rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, stream);
+  if (rc != FR_OK) return rc;
+  return fr_moe_down_combine(c.act, w2, c.topk_w, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, p.split_k, dtype, c.partial, out, stream);
 }
 
 extern "C" int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, const float* w1_scale, const void* w2q,
@@ -158,9 +176,7 @@ extern "C" int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, con
   FR_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FR_E_ALIGN, "fr_fused_moe_fp8: workspace must be 256-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
   Carve c = carve(workspace, M, H, F, E, topk, FR_FP8_E4M3, p);
-  rc = fr_gating_topk(logits, logits_dtype, M, E, E, topk, renormalize, c.topk_w, c.topk_ids, stream);
-  if (rc != FR_OK) return rc;
-  rc = fr_moe_align(c.topk_ids, FR_I32, M * topk, E, p.block, c.sorted, c.expert_ids, c.npost, c.align_ws, c.align_ws_bytes, stream);
+  rc = route_and_align(logits, logits_dtype, M, E, topk, renormalize, p.block, c, stream);
   if (rc != FR_OK) return rc;
   rc = quant_rows(x, x_dtype, M, nullptr, H, H, c.xq, c.x_scale, st);
   if (rc != FR_OK) return rc;

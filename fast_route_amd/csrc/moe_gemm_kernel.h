@@ -374,19 +374,21 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
       wsrc[ih] = static_cast<unsigned>((static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));
     }
-    // load q_ of an issuing wavefront (token-tile loads first, then weight-tile loads; the IW
-    // virtual wavefronts of one load index are adjacent) of tile tile_ into ring slot slot_
+    // load q_ of an issuing wavefront of tile tile_ into ring slot slot_.  Weight-tile loads come
+    // first: in the prologue they depend only on the expert id, so they are in flight while the
+    // sorted ids that the token-tile addresses need are still being fetched.  The IW virtual
+    // wavefronts of one load index are adjacent.
 #define FR_ISSUE_ONE(tile_, slot_, q_)                                                                     \
   {                                                                                                        \
     const int vw_ = wave_u + ((q_) % IW) * (NW / IW);                                                      \
-    if ((q_) < XI * IW) {                                                                                  \
+    if ((q_) < WI * IW) {                                                                                  \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
-          xrs, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + (((q_) / IW) * NW + vw_) * (kWave * 16)), 16,  \
-          xsrc[(q_) < XI * IW ? (q_) : 0], (tile_) * C::BKB, 0, 0);                                        \
+          wrs, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vw_) * (kWave * 16)), \
+          16, wsrc[(q_) < WI * IW ? (q_) : 0], (tile_) * C::BKB, 0, 0);                                    \
     } else {                                                                                               \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
-          wrs, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + ((((q_) - XI * IW) / IW) * NW + vw_) * (kWave * 16)), \
-          16, wsrc[(q_) < XI * IW ? 0 : (q_) - XI * IW], (tile_) * C::BKB, 0, 0);                          \
+          xrs, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WI * IW) / IW) * NW + vw_) * (kWave * 16)), \
+          16, xsrc[(q_) < WI * IW ? 0 : (q_) - WI * IW], (tile_) * C::BKB, 0, 0);                          \
     }                                                                                                      \
   }
 #define FR_ISSUE_PART(tile_, slot_, p_)                                                                    \

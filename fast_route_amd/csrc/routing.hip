@@ -10,7 +10,7 @@
 // the stable sort.  Small inputs run all three phases in one workgroup with the
 // tables in LDS; large ones use three launches (count, per-expert segment scan,
 // scatter + block table) and a global table.
-#include "fr_common.h"
+#include "gating_core.h"
 
 namespace fr {
 namespace {
@@ -156,6 +156,52 @@ __global__ __launch_bounds__(kSmallThreads) void align_small_kernel(
   segment_scatter(ids, lo, hi, E, bits_for(E), lane, &table[wave * E], sorted);
 }
 
+// Small batches, whole routing in one launch: the workgroup first gates every token
+// (a group of G lanes per token, 1024/G tokens per pass; weights and ids go to their
+// global arrays), then sorts the ids it has just written exactly as above.
+template <typename T, int G, int VPL>
+__global__ __launch_bounds__(kSmallThreads) void route_align_small_kernel(
+    const T* __restrict__ logits, int64_t M, int E, int topk, int renorm, int B, int seg_len, int64_t sorted_len,
+    float* __restrict__ w_out, int32_t* __restrict__ ids_out, int32_t* __restrict__ sorted,
+    int32_t* __restrict__ expert_ids, int32_t* __restrict__ npost_out) {
+  __shared__ int table[kSmallWaves * kSmallMaxE];
+  __shared__ int total[kSmallMaxE];
+  __shared__ int start[kSmallMaxE + 1];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  for (int i = tid; i < kSmallWaves * E; i += kSmallThreads) table[i] = 0;
+  constexpr int kPerPass = kSmallThreads / G;
+  for (int64_t base = 0; base < M; base += kPerPass) {  // uniform trip count: every lane joins the cross-lane ops
+    const int64_t token = base + tid / G;
+    const bool live = token < M;
+    const T* row = logits + (live ? token : 0) * E;
+    gate_token<G, VPL>([&](int e) { return to_float(row[e]); }, live, E, topk, renorm, w_out + token * topk,
+                       ids_out + token * topk);
+  }
+  __threadfence_block();
+  __syncthreads();  // the ids written above are read back below by other lanes of this workgroup
+  const int64_t n = M * topk;
+  const int64_t lo = min64(n, static_cast<int64_t>(wave) * seg_len);
+  const int64_t hi = min64(n, lo + seg_len);
+  segment_histogram(ids_out, lo, hi, E, lane, &table[wave * E]);
+  __syncthreads();
+  for (int e = tid; e < E; e += kSmallThreads) {
+    int running = 0;
+    for (int w = 0; w < kSmallWaves; ++w) {
+      const int c = table[w * E + e];
+      table[w * E + e] = running;
+      running += c;
+    }
+    total[e] = running;
+  }
+  __syncthreads();
+  if (wave == 0) scan_padded_totals(total, start, E, B, lane);
+  __syncthreads();
+  for (int i = tid; i < kSmallWaves * E; i += kSmallThreads) table[i] += start[i % E];
+  write_block_table(total, start, E, B, n, sorted_len, tid, kSmallThreads, sorted, expert_ids, npost_out);
+  __syncthreads();
+  segment_scatter(ids_out, lo, hi, E, bits_for(E), lane, &table[wave * E], sorted);
+}
+
 // ---------------------------------------------------------------- large path
 // counts is [E][S]: after align_segscan_kernel, counts[e][s] is the offset of
 // segment s inside expert e's run and totals[e] the length of the run.
@@ -270,7 +316,53 @@ int run(const void* ids_v, int64_t n, int E, int B, int32_t* sorted, int32_t* ex
   return check_launch("align kernels");
 }
 
+template <typename T, int G, int VPL>
+void launch_route_align(const void* logits, int64_t M, int E, int topk, int renorm, int B, int64_t sorted_len,
+                        float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, hipStream_t st) {
+  int seg_len = static_cast<int>(round_up(ceil_div(M * topk, kSmallWaves), kWave));
+  if (seg_len == 0) seg_len = kWave;
+  hipLaunchKernelGGL((route_align_small_kernel<T, G, VPL>), dim3(1), dim3(kSmallThreads), 0, st,
+                     static_cast<const T*>(logits), M, E, topk, renorm, B, seg_len, sorted_len, w, ids, sorted,
+                     expert_ids, npost);
+}
+
+template <typename T>
+void dispatch_route_align(const void* logits, int64_t M, int E, int topk, int renorm, int B, int64_t sorted_len,
+                          float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost,
+                          hipStream_t st) {
+#define FR_RA(G, VPL) launch_route_align<T, G, VPL>(logits, M, E, topk, renorm, B, sorted_len, w, ids, sorted, expert_ids, npost, st)
+  if (E <= 1) FR_RA(1, 1);
+  else if (E <= 2) FR_RA(2, 1);
+  else if (E <= 4) FR_RA(4, 1);
+  else if (E <= 8) FR_RA(8, 1);
+  else if (E <= 16) FR_RA(16, 1);
+  else if (E <= 32) FR_RA(32, 1);
+  else if (E <= 64) FR_RA(64, 1);
+  else if (E <= 128) FR_RA(64, 2);
+  else FR_RA(64, 4);
+#undef FR_RA
+}
+
 }  // namespace
+
+// Gating and routing arrays in one launch for small batches; false when the shape is
+// outside what one workgroup should do (the caller then runs the two stages separately).
+bool route_align_fits(int64_t M, int E, int topk) {
+  return M >= 1 && use_small_path(M * topk, E) && M * E <= 16384 && topk <= E;
+}
+int route_align_small(const void* logits, int logits_dtype, int64_t M, int E, int topk, int renorm, int block,
+                      float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost,
+                      hipStream_t st) {
+  const int64_t sorted_len = M * topk + int64_t(E) * (block - 1);
+  switch (logits_dtype) {
+    case FR_F32: dispatch_route_align<float>(logits, M, E, topk, renorm, block, sorted_len, w, ids, sorted, expert_ids, npost, st); break;
+    case FR_F16: dispatch_route_align<f16_t>(logits, M, E, topk, renorm, block, sorted_len, w, ids, sorted, expert_ids, npost, st); break;
+    case FR_BF16: dispatch_route_align<bf16_t>(logits, M, E, topk, renorm, block, sorted_len, w, ids, sorted, expert_ids, npost, st); break;
+    default: return fail(FR_E_DTYPE, "route_align_small: logits dtype %d not in {f32, f16, bf16}", logits_dtype);
+  }
+  return check_launch("route_align_small_kernel");
+}
+
 }  // namespace fr
 
 extern "C" int64_t fr_moe_align_workspace_bytes(int64_t n, int E) {
