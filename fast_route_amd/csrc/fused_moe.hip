@@ -81,7 +81,7 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   int block;
   if (avg <= 8) block = 16;
   else if (avg <= 32) block = 32;
-  else if (avg <= 384) block = 128;
+  else if (avg < 320) block = 128;
   else block = 256;
   // Down projection: N = H gives few feature tiles, so K is split.
   const int bf = block == 16 ? 64 : (block == 32 ? 128 : 256);
