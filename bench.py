@@ -143,6 +143,15 @@ def time_layer(torch, layer, steps, warmup):
         layer.fused()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # per-step spread (median, 20th and 80th percentile) from one event pair per step
+    pe = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in pe:
+        a.record()
+        layer.fused()
+        b.record()
+    torch.cuda.synchronize()
+    per = sorted(a.elapsed_time(b) * 1e3 for a, b in pe)
+    quant = {"p20": per[len(per) // 5], "p50": per[len(per) // 2], "p80": per[(4 * len(per)) // 5]}
     # per-stage times: the same kernels launched stage by stage with events on the launch stream
     evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(steps)]
     layer.staged()
@@ -153,14 +162,14 @@ def time_layer(torch, layer, steps, warmup):
     names = ["route", "moe_align", "moe_1+silu_and_mul", "moe_2+sum"]
     stage_us = {nm: sum(evs[s][i].elapsed_time(evs[s][i + 1]) for s in range(steps)) * 1e3 / steps
                 for i, nm in enumerate(names)}
-    return wall_ms, stage_us
+    return wall_ms, stage_us, quant
 
 
 def measure(torch, N, shape, M, w1, w2, steps, warmup, seed, fp8=None):
     layer = Layer(torch, N, shape, M, w1, w2, seed, fp8)
     if fp8:  # pad rows of act beyond npost are never written: keep them finite for the staged quantisation
         layer.act.zero_()
-    wall_ms, stage_us = time_layer(torch, layer, steps, warmup)
+    wall_ms, stage_us, quant = time_layer(torch, layer, steps, warmup)
     H, F, E, topk = shape["H"], shape["F"], shape["E"], shape["topk"]
     active = layer.active_experts()
     fl = layer_flops(M, H, F, topk)
@@ -170,7 +179,8 @@ def measure(torch, N, shape, M, w1, w2, steps, warmup, seed, fp8=None):
     t_hbm, t_mfma = by / (PEAK_HBM_GBS * 1e9), fl / (peak * 1e12)
     bound = "hbm" if t_hbm >= t_mfma else "mfma"
     rec = {
-        "tokens": M, "us_per_layer": round(wall_ms * 1e3, 2), "tflops": round(fl / t / 1e12, 3),
+        "tokens": M, "us_per_layer": round(wall_ms * 1e3, 2),
+        "us_per_layer_p20_p50_p80": [round(quant["p20"], 2), round(quant["p50"], 2), round(quant["p80"], 2)], "tflops": round(fl / t / 1e12, 3),
         "gbps": round(by / t / 1e9, 1), "active_experts": active, "bound": bound,
         "roofline_frac": round(max(t_hbm, t_mfma) / t, 4), "block": layer.plan.block, "split_k": layer.plan.split_k,
         "stage_us": {k: round(v, 2) for k, v in stage_us.items()},

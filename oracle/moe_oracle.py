@@ -240,7 +240,7 @@ def quant_e4m3_rows(x: torch.Tensor):
 
 
 def fused_moe_fp8(hidden_states, w1, w2, gating_output, topk: int, renormalize: bool = True):
-    """fp8 layer as BASELINE config 5 defines it: weights quantised per (expert,
+    """fp8 layer as the fp8 Mixtral workload defines it: weights quantised per (expert,
     output channel), activations per token (both before the gate/up GEMM and
     before the down GEMM), everything dequantised to fp32 and run through the
     fp32 oracle.  Returns (out fp32, dict with the quantised operands)."""

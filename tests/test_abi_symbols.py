@@ -61,7 +61,7 @@ def test_ops_refuse_cpu_tensors():
 
 
 def test_reference_import_paths_resolve():
-    """The reference's module paths (SURVEY: fast_route.layers.*, fast_route.ops.*) import here."""
+    """The reference's module paths (fast_route.layers.*, fast_route.ops.*) import here."""
     from fast_route.layers.stable_route import fused_moe as a
     from fast_route.layers.vllm_route import fused_moe as b
     from fast_route.layers.profile_fused_route import fused_moe as c

@@ -41,7 +41,7 @@ def _inputs(M, H, Fd, E, seed, dtype, zipf=False):
 @pytest.mark.parametrize("M", [1, 16, 64, 200, 512, 2048])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_small_layer_config(native, M, dtype):
-    """BASELINE config 1 (H1024 F3584 E8 top2) at token counts that hit every tile plan."""
+    """Small layer (H1024 F3584 E8 top2) at token counts that hit every tile plan."""
     from fast_route_amd import fused_moe
     _say(f"layer C1 M={M} dtype={dtype}")
     x, logits, w1, w2 = _inputs(M, 1024, 3584, 8, 1337, dtype)
@@ -53,7 +53,7 @@ def test_small_layer_config(native, M, dtype):
 
 @pytest.mark.parametrize("M", [1, 32, 128, 700])
 def test_fine_grained_config(native, M):
-    """BASELINE config 4 shape family (E64 top6, Zipf-skewed load), reduced H/F for CPU oracle time."""
+    """Fine-grained many-expert shape family (E64 top6, Zipf-skewed load), reduced H/F for CPU oracle time."""
     from fast_route_amd import fused_moe
     _say(f"layer C4-like M={M}")
     x, logits, w1, w2 = _inputs(M, 512, 384, 64, 99, torch.bfloat16, zipf=True)
@@ -232,7 +232,7 @@ def test_transformer_layer_bench_runs_and_matches_its_parts(native):
 
 
 def test_mixtral_shape_sampled_tokens_and_properties(native):
-    """BASELINE config 2 at full size (H4096 F14336 E8 top2): oracle on a sample of
+    """Mixtral-8x7B shape at full size (H4096 F14336 E8 top2): oracle on a sample of
     tokens, plus size-independent properties on all of them."""
     from fast_route_amd import fused_moe, fused_experts
     dtype = torch.bfloat16
