@@ -28,6 +28,34 @@ __global__ __launch_bounds__(kGateThreads) void gating_topk_kernel(
   }
 }
 
+// 4 consecutive logits as fp32 from a 4-element-aligned address
+template <typename T>
+__device__ __forceinline__ f32x4 load4_as_float(const T* p) {
+  if constexpr (sizeof(T) == 4) {
+    return *reinterpret_cast<const f32x4*>(p);
+  } else {
+    typedef T vec4 __attribute__((ext_vector_type(4)));
+    const vec4 t = *reinterpret_cast<const vec4*>(p);
+    return f32x4{to_float(t[0]), to_float(t[1]), to_float(t[2]), to_float(t[3])};
+  }
+}
+
+template <typename T, int G, int NV>
+__global__ __launch_bounds__(kGateThreads) void gating_topk_blocked_kernel(
+    const T* __restrict__ logits, int64_t M, int E, int64_t ld, int topk, int renorm,
+    float* __restrict__ w_out, int32_t* __restrict__ ids_out) {
+  constexpr int64_t kPerBlock = kGateThreads / G;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kPerBlock;
+  const int64_t rounds = (M + stride - 1) / stride;  // uniform trip count: every lane joins the cross-lane ops
+  int64_t token = static_cast<int64_t>(blockIdx.x) * kPerBlock + threadIdx.x / G;
+  for (int64_t it = 0; it < rounds; ++it, token += stride) {
+    const bool live = token < M;
+    const T* row = logits + (live ? token : 0) * ld;
+    gate_token_blocked<G, NV>([&](int e0) { return load4_as_float(row + e0); }, live, E, topk, renorm,
+                              w_out + token * topk, ids_out + token * topk);
+  }
+}
+
 // ---- gate-matrix form: logits tile by MFMA, then the same gating -------------
 // One workgroup owns kRgTokens tokens (16 per wavefront).  The gate matrix is
 // [H, E] with experts contiguous, so each K tile of it is transposed through
@@ -121,9 +149,30 @@ void launch(const void* logits, int64_t M, int E, int64_t ld, int topk, int reno
                      static_cast<const T*>(logits), M, E, ld, topk, renorm, w, ids);
 }
 
+template <typename T, int G, int NV>
+void launch_blocked(const void* logits, int64_t M, int E, int64_t ld, int topk, int renorm, float* w,
+                    int32_t* ids, hipStream_t st) {
+  const int64_t tokens_per_block = kGateThreads / G;
+  int64_t blocks = ceil_div(M, tokens_per_block);
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL((gating_topk_blocked_kernel<T, G, NV>), dim3(static_cast<unsigned>(blocks)), dim3(kGateThreads), 0,
+                     st, static_cast<const T*>(logits), M, E, ld, topk, renorm, w, ids);
+}
+
 template <typename T>
 int dispatch(const void* logits, int64_t M, int E, int64_t ld, int topk, int renorm, float* w,
              int32_t* ids, hipStream_t st) {
+  // many experts, rows that 4-element vector loads can read: few lanes per token
+  const bool vec_ok = E > 16 && E % 4 == 0 && ld % 4 == 0 &&
+                      (reinterpret_cast<uintptr_t>(logits) % (4 * sizeof(T))) == 0;
+  const int lanes = E <= 64 ? 4 : (E <= 128 ? 8 : 16);
+  if (vec_ok && topk <= kBlockedSlots * lanes) {
+    if (E <= 32) launch_blocked<T, 4, 2>(logits, M, E, ld, topk, renorm, w, ids, st);
+    else if (E <= 64) launch_blocked<T, 4, 4>(logits, M, E, ld, topk, renorm, w, ids, st);
+    else if (E <= 128) launch_blocked<T, 8, 4>(logits, M, E, ld, topk, renorm, w, ids, st);
+    else launch_blocked<T, 16, 4>(logits, M, E, ld, topk, renorm, w, ids, st);
+    return check_launch("gating_topk_blocked_kernel");
+  }
   if (E <= 1) launch<T, 1, 1>(logits, M, E, ld, topk, renorm, w, ids, st);
   else if (E <= 2) launch<T, 2, 1>(logits, M, E, ld, topk, renorm, w, ids, st);
   else if (E <= 4) launch<T, 4, 1>(logits, M, E, ld, topk, renorm, w, ids, st);

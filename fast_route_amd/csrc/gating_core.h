@@ -148,7 +148,7 @@ __device__ __forceinline__ void gate_token(Load load, bool live, int E, int topk
   }
   unsigned taken = 0;
   float sel_sum = 0.f;
-  const unsigned vkey = float_key(v[0]);
+  const unsigned vkey = float_key(v[0] + 0.f);  // + 0.f: -0 and +0 are the same value
   for (int r = 0; r < topk; ++r) {
     float bv;
     int bi;
@@ -190,6 +190,109 @@ __device__ __forceinline__ void gate_token(Load load, bool live, int E, int topk
   if (live) {
 #pragma unroll
     for (int sl = 0; sl < VPL; ++sl) {
+      const int r = sl * G + g;
+      if (r < topk) {
+        w_row[r] = __expf(sel_v[sl] - m) / denom;
+        id_row[r] = sel_i[sl];
+      }
+    }
+  }
+}
+
+// Many experts: a group of only G lanes owns a token and every lane keeps NV vectors of 4
+// consecutive logits, vector j of lane g holding experts 4*(G*j + g) .. 4*(G*j + g) + 3, so
+// the G lanes read 4*G consecutive logits of the token per load and a wavefront gates 64/G
+// tokens at once: the cross-lane rounds (the cost of the one-logit-per-lane form, a wavefront
+// instruction per step per token) shrink to log2(G) steps shared by 64/G tokens.  Inside a
+// lane expert indices rise with the slot number, across lanes ties go to the lower index,
+// so the order is still (value descending, index ascending).  load4(e0) returns logits
+// e0..e0+3; E must be a multiple of 4.
+constexpr int kBlockedSlots = 4;  // result slots per lane: topk <= kBlockedSlots * G
+
+template <int G, int NV, typename Load4>
+__device__ __forceinline__ void gate_token_blocked(Load4 load4, bool live, int E, int topk, int renorm,
+                                                   float* __restrict__ w_row, int32_t* __restrict__ id_row) {
+  constexpr int VPL = 4 * NV;
+  static_assert(G <= 16, "the all-reduce uses the in-row DPP steps only");
+  const int g = threadIdx.x % G;
+  float v[VPL];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int e0 = 4 * (G * j + g);
+    f32x4 t = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    if (live && e0 < E) t = load4(e0);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) v[4 * j + c] = t[c];
+  }
+  float m = v[0];
+  float s = (v[0] == -INFINITY) ? 0.f : 1.f;
+#pragma unroll
+  for (int i = 1; i < VPL; ++i) {
+    if (v[i] == -INFINITY) continue;
+    const float mn = fmaxf(m, v[i]);
+    s = (m == -INFINITY ? 0.f : s * __expf(m - mn)) + __expf(v[i] - mn);
+    m = mn;
+  }
+  group_online_softmax<G>(m, s);
+
+  // Order keys of this lane's logits (0 = not a candidate).  Inside the lane a strict
+  // "greater" scan keeps the lowest slot, i.e. the lowest expert index, among equal keys.
+  unsigned k[VPL];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int e = 4 * (G * (i / 4) + g) + (i % 4);
+    k[i] = (e < E) ? float_key(v[i] + 0.f) : 0u;  // + 0.f: -0 and +0 are the same value
+  }
+  float sel_v[kBlockedSlots];
+  int sel_i[kBlockedSlots];
+#pragma unroll
+  for (int i = 0; i < kBlockedSlots; ++i) {
+    sel_v[i] = -INFINITY;
+    sel_i[i] = 0;
+  }
+  int last = -1;  // slot this lane gave away in the previous round
+  float sel_sum = 0.f;
+  for (int r = 0; r < topk; ++r) {
+    unsigned bk = 0u;
+    int bs = 0;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      if (i == last) k[i] = 0u;
+      if (k[i] > bk) {
+        bk = k[i];
+        bs = i;
+      }
+    }
+    int be = 4 * (G * (bs >> 2) + g) + (bs & 3);
+    // all-reduce over the group: larger key wins, equal keys go to the lower expert index
+    auto step = [&](auto tag) {
+      constexpr int S = decltype(tag)::value;
+      const unsigned ok = static_cast<unsigned>(partner_i32<S>(static_cast<int>(bk)));
+      const int oe = partner_i32<S>(be);
+      if (ok > bk || (ok == bk && oe < be)) {
+        bk = ok;
+        be = oe;
+      }
+    };
+    if constexpr (G > 1) step(std::integral_constant<int, 1>{});
+    if constexpr (G > 2) step(std::integral_constant<int, 2>{});
+    if constexpr (G > 4) step(std::integral_constant<int, 4>{});
+    if constexpr (G > 8) step(std::integral_constant<int, 8>{});
+    last = ((be >> 2) % G == g) ? (4 * (be / (4 * G)) + (be & 3)) : -1;
+    const float bv = key_float(bk);
+    sel_sum += __expf(bv - m);
+#pragma unroll
+    for (int sl = 0; sl < kBlockedSlots; ++sl) {
+      if (r == sl * G + g) {
+        sel_v[sl] = bv;
+        sel_i[sl] = be;
+      }
+    }
+  }
+  const float denom = renorm ? sel_sum : s;
+  if (live) {
+#pragma unroll
+    for (int sl = 0; sl < kBlockedSlots; ++sl) {
       const int r = sl * G + g;
       if (r < topk) {
         w_row[r] = __expf(sel_v[sl] - m) / denom;

@@ -47,6 +47,7 @@ def test_gating_ties_and_special_rows(native):
         [-30.0, -30.0, -30.0, -30.0, -30.0, 30.0, -30.0, -30.0],
         [5.0, 4.0, 3.0, 2.0, 1.0, 0.0, -1.0, -2.0],
         [-2.0, -1.0, 0.0, 1.0, 2.0, 3.0, 4.0, 5.0],
+        [-0.0, 0.0, -0.0, 0.0, -1.0, 0.0, -0.0, -1.0],  # signed zeros are one value: ties by index
     ]
     logits = torch.tensor(rows)
     for k in (1, 2, 4, 8):
@@ -57,6 +58,30 @@ def test_gating_ties_and_special_rows(native):
             torch.testing.assert_close(w, rw, atol=W_ATOL, rtol=0)
     w, ids = _run_gating(logits.cuda(), 4, True)
     assert ids[0].tolist() == [0, 1, 2, 3] and ids[1].tolist() == [1, 2, 4, 0]
+
+
+@pytest.mark.parametrize("E,topk", [(32, 5), (64, 6), (64, 16), (64, 40), (128, 8), (256, 8), (48, 3)])
+def test_gating_ties_many_experts(native, E, topk):
+    """Rows built from a handful of distinct values, so every round of the selection has
+    ties inside a lane, across lanes and across the vectors of a lane; +0 / -0 tie too.
+    (topk = 40 exceeds the result slots of the few-lanes-per-token form: fallback path.)"""
+    _say(f"gating ties E={E} topk={topk}")
+    g = torch.Generator().manual_seed(E * 131 + topk)
+    vals = torch.tensor([0.0, -0.0, 1.5, -1.5, 3.0, 0.25])
+    logits = vals[torch.randint(0, len(vals), (257, E), generator=g)]
+    logits[0] = 0.0
+    logits[1] = torch.arange(E, dtype=torch.float32) % 3
+    logits[2] = -torch.arange(E, dtype=torch.float32)
+    for renorm in (True, False):
+        w, ids = _run_gating(logits.cuda(), topk, renorm)
+        rw, rid = oracle.gating_topk(logits, topk, renorm)
+        assert torch.equal(ids, rid)
+        torch.testing.assert_close(w, rw, atol=W_ATOL, rtol=0)
+    # a row stride that is not a multiple of 4 takes the one-logit-per-lane path
+    wide = torch.zeros(257, E + 3)
+    wide[:, :E] = logits
+    w2, ids2 = _run_gating(wide.cuda()[:, :E], topk, True)
+    assert torch.equal(ids2, oracle.gating_topk(logits, topk, True)[1])
 
 
 def test_gating_reference_route_test_recipe(native):
