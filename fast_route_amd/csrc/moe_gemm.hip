@@ -42,7 +42,7 @@ template <typename T> struct Tiles {  // bf16 / fp16
   typedef Cfg<32, 128, 128, 1, 4, 16, 2, 3> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
   typedef Cfg<32, 128, 512, 1, 4, 16, 1, 2> T32L;
-  typedef Cfg<16, 128, 512, 1, 4, 16, 1, 2> T16L;
+  typedef Cfg<16, 64, 512, 1, 2, 16, 2, 2> T16L;
 };
 template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per two K-steps
   typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
@@ -51,7 +51,7 @@ template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per
   typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
   typedef Cfg<32, 128, 512, 1, 4, 16, 1, 2> T32L;
-  typedef Cfg<16, 128, 512, 1, 4, 16, 1, 2> T16L;
+  typedef Cfg<16, 64, 512, 1, 2, 16, 2, 2> T16L;
 };
 
 bool valid_block(int block) { return block == 16 || block == 32 || block == 64 || block == 128 || block == 256; }
