@@ -166,7 +166,8 @@ int dispatch(const void* logits, int64_t M, int E, int64_t ld, int topk, int ren
   const bool vec_ok = E > 16 && E % 4 == 0 && ld % 4 == 0 &&
                       (reinterpret_cast<uintptr_t>(logits) % (4 * sizeof(T))) == 0;
   const int lanes = E <= 64 ? 4 : (E <= 128 ? 8 : 16);
-  if (vec_ok && topk <= kBlockedSlots * lanes) {
+  // (a short batch is latency bound: one logit per lane finishes a token in fewer dependent steps)
+  if (vec_ok && M >= 1024 && topk <= kBlockedSlots * lanes) {
     if (E <= 32) launch_blocked<T, 4, 2>(logits, M, E, ld, topk, renorm, w, ids, st);
     else if (E <= 64) launch_blocked<T, 4, 4>(logits, M, E, ld, topk, renorm, w, ids, st);
     else if (E <= 128) launch_blocked<T, 8, 4>(logits, M, E, ld, topk, renorm, w, ids, st);

@@ -29,7 +29,7 @@ def _run_gating(logits_dev, topk, renorm):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("renorm", [True, False])
 def test_gating_parity(native, E, topk, dtype, renorm):
-    for M in (1, 63, 1000):
+    for M in (1, 63, 1000, 2500):
         _say(f"gating E={E} k={topk} dtype={dtype} renorm={renorm} M={M}")
         g = torch.Generator().manual_seed(E * 131 + topk * 7 + M)
         logits = torch.randn(M, E, generator=g).to(dtype)  # bf16/fp16 rounding creates exact ties
@@ -68,7 +68,7 @@ def test_gating_ties_many_experts(native, E, topk):
     _say(f"gating ties E={E} topk={topk}")
     g = torch.Generator().manual_seed(E * 131 + topk)
     vals = torch.tensor([0.0, -0.0, 1.5, -1.5, 3.0, 0.25])
-    logits = vals[torch.randint(0, len(vals), (257, E), generator=g)]
+    logits = vals[torch.randint(0, len(vals), (1300, E), generator=g)]  # long enough for the few-lanes-per-token form
     logits[0] = 0.0
     logits[1] = torch.arange(E, dtype=torch.float32) % 3
     logits[2] = -torch.arange(E, dtype=torch.float32)
@@ -78,7 +78,7 @@ def test_gating_ties_many_experts(native, E, topk):
         assert torch.equal(ids, rid)
         torch.testing.assert_close(w, rw, atol=W_ATOL, rtol=0)
     # a row stride that is not a multiple of 4 takes the one-logit-per-lane path
-    wide = torch.zeros(257, E + 3)
+    wide = torch.zeros(1300, E + 3)
     wide[:, :E] = logits
     w2, ids2 = _run_gating(wide.cuda()[:, :E], topk, True)
     assert torch.equal(ids2, oracle.gating_topk(logits, topk, True)[1])
