@@ -74,3 +74,29 @@ def test_reference_import_paths_resolve():
     assert list(inspect.signature(fused_route).parameters) == ["hidden_state", "gate", "topk", "topk_weights", "topk_ids", "renormalize"]
     assert list(inspect.signature(moe_align_block_size).parameters) == ["topk_ids", "block_size", "num_experts"]
     assert list(inspect.signature(invoke_fused_moe_kernel).parameters)[:4] == ["A", "B", "C", "topk_weights"]
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py is single-GPU: any other --gpus value exits with a message that says so."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "single-GPU" in r.stderr
+
+
+def test_recorded_traffic_matches_profiles_file():
+    """bench.py reports roofline.traffic from profiles/hbm_traffic.json for the workloads recorded there."""
+    import importlib.util
+    import json
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_mod", os.path.join(root, "bench.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    rec = json.load(open(os.path.join(root, "profiles", "hbm_traffic.json")))
+    key = "moe_layer_tflops_mixtral_bf16_M4096"
+    assert mod.recorded_traffic(key) == rec[key]["traffic_bytes"] == rec[key]["fetch_bytes"] + rec[key]["write_bytes"]
+    assert mod.recorded_traffic("no_such_workload") is None
