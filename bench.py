@@ -198,13 +198,15 @@ def kernel_roofline(shape, rec, fp8=False):
     eb = 1 if fp8 else 2
     byts = rec["active_experts"] * 2 * F * H * eb + M * H * eb + M * topk * F * 2
     peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
+    # 256-row routing blocks of 2-byte operands run the persistent form of the kernel
+    name = ("moe_gemm_persistent_kernel" if rec["block"] == 256 and not fp8 else "moe_gemm_kernel") + "<EPI_SILU>"
     if flops / (peak * 1e12) >= byts / (PEAK_HBM_GBS * 1e9):
         ach = flops / dur / 1e12
-        return {"kernel": "moe_gemm_kernel<EPI_SILU>", "bound": "mfma", "achieved": round(ach, 2), "peak": peak,
+        return {"kernel": name, "bound": "mfma", "achieved": round(ach, 2), "peak": peak,
                 "unit": "TFLOP/s", "frac": round(ach / peak, 4), "traffic": None,
                 "avg_launch_us": round(dur * 1e6, 2), "algorithmic_flops_per_launch": flops}
     ach = byts / dur / 1e9
-    return {"kernel": "moe_gemm_kernel<EPI_SILU>", "bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
+    return {"kernel": name, "bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
             "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
             "avg_launch_us": round(dur * 1e6, 2), "algorithmic_bytes_per_launch": byts}
 

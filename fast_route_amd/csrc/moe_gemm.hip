@@ -1,5 +1,5 @@
 // Host side of the grouped expert GEMMs: tile selection, launches, top-k combine.
-#include "moe_gemm_kernel.h"
+#include "moe_gemm_persistent.h"
 
 namespace fr {
 
@@ -71,7 +71,12 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
     a.k_per_split = static_cast<int>(round_up(ceil_div(a.K, splits), bk));
   };
   switch (block) {
-    case 256: fill(256, TL::T256::BF, TL::T256::BKB); return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
+    case 256:
+      fill(256, TL::T256::BF, TL::T256::BKB);
+      // One workgroup per CU: the persistent form hides each tile's ring fill and drain behind
+      // its neighbour's.  The fp8 fragments leave no registers for the second address set.
+      if constexpr (sizeof(T) == 2) return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
+      else return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
     case 128: fill(128, TL::T128::BF, TL::T128::BKB); return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
     case 64: fill(64, TL::T64::BF, TL::T64::BKB); return launch_gemm<T, typename TL::T64, EPI>(a, splits, st);
     case 32:

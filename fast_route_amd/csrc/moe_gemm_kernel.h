@@ -139,6 +139,108 @@ __device__ __forceinline__ int swizzle(int row, int chunk) {
   return chunk ^ ((row / ROWS_PER_LINE) & MASK);
 }
 
+// Epilogue of one tile: the lane holds token column (lane % TILE) of each token tile of its
+// wavefront and, per accumulator group, 4 consecutive features.
+#if defined(__HIP_DEVICE_COMPILE__)
+// Buffer resource over the whole address space from `p` on.  The pointer is the same in every
+// lane; reading it through the first lane tells the compiler so, which otherwise may keep the
+// resource in vector registers and wrap each load in a loop over the distinct lane values.
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_rsrc(const T* p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint64_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(v))));
+  const uint64_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(v >> 32))));
+  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(hi << 32 | lo), 0, -1, 0x00020000);
+}
+#endif
+
+template <typename T, typename C, int EPI, typename AccT>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::JF][C::IT], int pid_t, int pid_f,
+                                              int expert, int split, int wt, int wf, int frow, int kgrp) {
+  typedef Elem<T> E;
+  typedef typename E::out_t out_t;
+  typedef typename E::out4 out4;
+  constexpr int BT = C::BT, BF = C::BF;
+  constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
+  // ---- epilogue -------------------------------------------------------------
+  // lane holds token column (lane % TILE) of each token tile and, per accumulator
+  // group g (TILE==32: 4 groups of 4 regs; TILE==16: one), 4 consecutive features
+  // starting at g*8 + kgrp*4 (TILE==32) or kgrp*4 (TILE==16) inside the MFMA tile.
+  constexpr int GROUPS = ACC_N / 4;
+  const float* wsc = nullptr;
+  if constexpr (E::SCALED) wsc = a.w_scale + static_cast<int64_t>(expert) * a.w_rows;
+#pragma unroll
+  for (int i = 0; i < C::IT; ++i) {
+    const int slot = pid_t * BT + wt * C::TT + i * C::TILE + frow;
+    int sid = 0;
+    if constexpr (EPI != EPI_SILU || E::SCALED) sid = a.sorted[slot];
+    float xs = 1.f;
+    if constexpr (E::SCALED) {
+      if (a.top_k > 0) xs = sid < a.num_valid ? a.x_scale[sid / a.top_k] : 1.f;
+      else xs = a.x_scale[slot];
+    }
+    if constexpr (EPI == EPI_SILU) {
+      constexpr int HJ = C::JF / 2;
+      out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(slot) * a.ldo;
+#pragma unroll
+      for (int j = 0; j < HJ; ++j)
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+          const int f = pid_f * (BF / 2) + wf * (C::TF / 2) + j * C::TILE + g * 8 + kgrp * 4;
+          out4 o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float gv = acc[j][i][g * 4 + r], uv = acc[j + HJ][i][g * 4 + r];
+            if constexpr (E::SCALED) {
+              const int fc = f + r < a.N ? f + r : a.N - 1;
+              gv *= xs * wsc[fc];
+              uv *= xs * wsc[a.N + fc];
+            }
+            o[r] = static_cast<out_t>(silu(gv) * uv);
+          }
+          if (f + 3 < a.N) *reinterpret_cast<out4*>(orow + f) = o;
+          else
+            for (int r = 0; r < 4; ++r)
+              if (f + r < a.N) orow[f + r] = o[r];
+        }
+    } else {
+      if (sid < a.num_valid) {
+        const float rw = (a.mul_weight ? a.topk_w[sid] : 1.f) * xs;
+#pragma unroll
+        for (int j = 0; j < C::JF; ++j)
+#pragma unroll
+          for (int g = 0; g < GROUPS; ++g) {
+            const int f = pid_f * BF + wf * C::TF + j * C::TILE + g * 8 + kgrp * 4;
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              v[r] = acc[j][i][g * 4 + r] * rw;
+              if constexpr (E::SCALED) v[r] *= wsc[f + r < a.N ? f + r : a.N - 1];
+            }
+            if constexpr (EPI == EPI_DOWN) {
+              float* orow = static_cast<float*>(a.out) + static_cast<int64_t>(split) * a.split_stride +
+                            static_cast<int64_t>(sid) * a.ldo;
+              const f32x4 o = {v[0], v[1], v[2], v[3]};
+              if (f + 3 < a.N) *reinterpret_cast<f32x4*>(orow + f) = o;
+              else
+                for (int r = 0; r < 4; ++r)
+                  if (f + r < a.N) orow[f + r] = v[r];
+            } else {
+              out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(sid) * a.ldo;
+              out4 o;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) o[r] = static_cast<out_t>(v[r]);
+              if (f + 3 < a.N) *reinterpret_cast<out4*>(orow + f) = o;
+              else
+                for (int r = 0; r < 4; ++r)
+                  if (f + r < a.N) orow[f + r] = o[r];
+            }
+          }
+      }
+    }
+  }
+}
+
 template <typename T, typename C, int EPI>
 __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs a) {
   typedef Elem<T> E;
@@ -356,8 +458,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     // first row; gathered rows and an expert's weights must span less than 4 GiB
     // (checked by the launcher).
     const int64_t xrow0 = a.top_k > 0 ? 0 : static_cast<int64_t>(pid_t) * BT;
-    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(X + xrow0 * a.ldx), 0, -1, 0x00020000);
-    const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(W), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrs = uniform_rsrc(X + xrow0 * a.ldx);
+    const __amdgpu_buffer_rsrc_t wrs = uniform_rsrc(W);
     const bool issuer = wave_u < NW / IW;
     unsigned xsrc[XI * IW], wsrc[WI * IW];  // byte offsets, [load][virtual wavefront]
 #pragma unroll
@@ -500,83 +602,7 @@ _Pragma("unroll") \
 #undef FR_READ_FRAGS
 #undef FR_MMA
 
-  // ---- epilogue -------------------------------------------------------------
-  // lane holds token column (lane % TILE) of each token tile and, per accumulator
-  // group g (TILE==32: 4 groups of 4 regs; TILE==16: one), 4 consecutive features
-  // starting at g*8 + kgrp*4 (TILE==32) or kgrp*4 (TILE==16) inside the MFMA tile.
-  constexpr int GROUPS = ACC_N / 4;
-  const float* wsc = nullptr;
-  if constexpr (E::SCALED) wsc = a.w_scale + static_cast<int64_t>(expert) * a.w_rows;
-#pragma unroll
-  for (int i = 0; i < C::IT; ++i) {
-    const int slot = pid_t * BT + wt * C::TT + i * C::TILE + frow;
-    int sid = 0;
-    if constexpr (EPI != EPI_SILU || E::SCALED) sid = a.sorted[slot];
-    float xs = 1.f;
-    if constexpr (E::SCALED) {
-      if (a.top_k > 0) xs = sid < a.num_valid ? a.x_scale[sid / a.top_k] : 1.f;
-      else xs = a.x_scale[slot];
-    }
-    if constexpr (EPI == EPI_SILU) {
-      constexpr int HJ = C::JF / 2;
-      out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(slot) * a.ldo;
-#pragma unroll
-      for (int j = 0; j < HJ; ++j)
-#pragma unroll
-        for (int g = 0; g < GROUPS; ++g) {
-          const int f = pid_f * (BF / 2) + wf * (C::TF / 2) + j * C::TILE + g * 8 + kgrp * 4;
-          out4 o;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            float gv = acc[j][i][g * 4 + r], uv = acc[j + HJ][i][g * 4 + r];
-            if constexpr (E::SCALED) {
-              const int fc = f + r < a.N ? f + r : a.N - 1;
-              gv *= xs * wsc[fc];
-              uv *= xs * wsc[a.N + fc];
-            }
-            o[r] = static_cast<out_t>(silu(gv) * uv);
-          }
-          if (f + 3 < a.N) *reinterpret_cast<out4*>(orow + f) = o;
-          else
-            for (int r = 0; r < 4; ++r)
-              if (f + r < a.N) orow[f + r] = o[r];
-        }
-    } else {
-      if (sid < a.num_valid) {
-        const float rw = (a.mul_weight ? a.topk_w[sid] : 1.f) * xs;
-#pragma unroll
-        for (int j = 0; j < C::JF; ++j)
-#pragma unroll
-          for (int g = 0; g < GROUPS; ++g) {
-            const int f = pid_f * BF + wf * C::TF + j * C::TILE + g * 8 + kgrp * 4;
-            float v[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              v[r] = acc[j][i][g * 4 + r] * rw;
-              if constexpr (E::SCALED) v[r] *= wsc[f + r < a.N ? f + r : a.N - 1];
-            }
-            if constexpr (EPI == EPI_DOWN) {
-              float* orow = static_cast<float*>(a.out) + static_cast<int64_t>(split) * a.split_stride +
-                            static_cast<int64_t>(sid) * a.ldo;
-              const f32x4 o = {v[0], v[1], v[2], v[3]};
-              if (f + 3 < a.N) *reinterpret_cast<f32x4*>(orow + f) = o;
-              else
-                for (int r = 0; r < 4; ++r)
-                  if (f + r < a.N) orow[f + r] = v[r];
-            } else {
-              out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(sid) * a.ldo;
-              out4 o;
-#pragma unroll
-              for (int r = 0; r < 4; ++r) o[r] = static_cast<out_t>(v[r]);
-              if (f + 3 < a.N) *reinterpret_cast<out4*>(orow + f) = o;
-              else
-                for (int r = 0; r < 4; ++r)
-                  if (f + r < a.N) orow[f + r] = o[r];
-            }
-          }
-      }
-    }
-  }
+  gemm_epilogue<T, C, EPI>(a, acc, pid_t, pid_f, expert, split, wt, wf, frow, kgrp);
 }
 
 template <typename T, typename C, int EPI>

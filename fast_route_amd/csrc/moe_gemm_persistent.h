@@ -1,0 +1,319 @@
+// Persistent form of the direct-to-LDS grouped GEMM: one workgroup per resident slot walks
+// several tiles, and the LDS ring never drains between them.  While the last K tiles of
+// one output tile are being multiplied, the ring is already refilled with the first K
+// tiles of the workgroup's next output tile (whose routing data was fetched a whole tile
+// earlier), so the start-up of a tile (dependent loads of block table, sorted ids, first
+// operand tiles) and the memory side of its epilogue hide behind MFMA work.  It pays for
+// tiles that leave room for one workgroup per CU only (256 x 256); smaller tiles already
+// overlap one workgroup's start-up with the other's MFMAs.
+//
+// Same tile shapes, LDS layout, swizzle, fragment double buffering, barrier placement and
+// epilogues as moe_gemm_kernel (STAGES >= 2, refill in one group); see there.
+#pragma once
+#include "moe_gemm_kernel.h"
+
+namespace fr {
+
+template <typename T, typename C, int EPI>
+__global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(const GemmArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)  // buffer resources and LDS-DMA builtins exist in the device pass only
+  typedef Elem<T> E;
+  typedef typename std::conditional<C::TILE == 32, f32x16, f32x4>::type acc_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  constexpr int BT = C::BT, BF = C::BF, CPR = C::CPR, FC = E::FC;
+  constexpr int EPC = 16 / static_cast<int>(sizeof(T));
+  constexpr int BK = C::BKB / static_cast<int>(sizeof(T));
+  constexpr int KS = CPR / (C::KGROUPS * FC);
+  constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
+  constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, IW = C::IW, NLI = (XI + WI) * IW;
+  constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
+  static_assert(S >= 2 && C::SPREAD <= 1, "persistent form: ring of at least two slots, refill in one group");
+  static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
+  static_assert((S - 1) * NLI <= 63, "vmcnt budget");
+  static_assert(EPI != EPI_SILU || C::JF % 2 == 0, "gate and up tiles must pair up inside a wave");
+  static_assert(IW >= 1 && NW % IW == 0, "issue width");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  u32x4* lds = reinterpret_cast<u32x4*>(lds_raw);
+  constexpr int WBASE = S * C::XCH;  // LDS map (16-byte units): X slots first, then W slots
+
+  // ---- schedule ---------------------------------------------------------------
+  // The real tile count is dealt to the 8 XCDs (workgroup id mod 8) in contiguous ranges; the
+  // workgroups of one XCD take the tiles of its range round robin, so at any moment they work on
+  // consecutive tiles (group_t token blocks x consecutive feature tiles: shared in that XCD's L2).
+  const int npost = a.npost[0];
+  const int nt = min(npost / BT, a.num_t_blocks);
+  const int total = nt * a.num_f_tiles;
+  const int xcd = blockIdx.x & 7, nper = gridDim.x >> 3;
+  const int per = total >> 3, rem = total & 7;
+  const int xbase = xcd * per + (xcd < rem ? xcd : rem), xcount = per + (xcd < rem ? 1 : 0);
+  int loc = blockIdx.x >> 3;
+  if (loc >= xcount) return;
+  const int in_group = a.group_t * a.num_f_tiles;
+  const int split = blockIdx.y;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wt = wave / C::WF, wf = wave % C::WF;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const bool issuer = wave_u < NW / IW;
+  const T* X = static_cast<const T*>(a.X);
+  const int k0 = split * a.k_per_split;
+  const int k_tiles = min(a.k_per_split, a.K - k0) / BK;  // >= S + 2 (checked by the launcher)
+
+#define FR_COORDS(lin_, pt_, pf_)                                  \
+  {                                                                \
+    const int gid_ = (lin_) / in_group, first_ = gid_ * a.group_t; \
+    const int gsz_ = min(nt - first_, a.group_t);                  \
+    pt_ = first_ + ((lin_) % in_group) % gsz_;                     \
+    pf_ = ((lin_) % in_group) / gsz_;                              \
+  }
+  // rows of the load slots this wavefront issues: load index ih -> tile row
+#define FR_SLOT_ROW(ih_, rr_, c_)                                                  \
+  const int vw_ = (wave_u + ((ih_) % IW) * (NW / IW)) % NW;                        \
+  const int slot_ = (((ih_) / IW) * NW + vw_) * kWave + lane;                      \
+  const int rr_ = slot_ / CPR, c_ = swizzle<CPR>(rr_, slot_ % CPR);
+  auto w_src_row = [&](int pf, int rr) -> int {
+    if constexpr (EPI == EPI_SILU) {
+      const int half = rr / (BF / 2), f = pf * (BF / 2) + rr % (BF / 2);
+      return half * a.N + (f < a.N ? f : a.N - 1);
+    } else {
+      const int f = pf * BF + rr;
+      return f < a.N ? f : a.N - 1;
+    }
+  };
+
+  // ---- per-lane fragment rows ---------------------------------------------------
+  const int frow = lane % C::TILE, kgrp = lane / C::TILE;
+  int xoff[C::IT], woff[C::JF], xkey[C::IT], wkey[C::JF];
+#pragma unroll
+  for (int i = 0; i < C::IT; ++i) {
+    const int r = wt * C::TT + i * C::TILE + frow;
+    xoff[i] = r * CPR;
+    xkey[i] = swizzle<CPR>(r, 0);
+  }
+#pragma unroll
+  for (int j = 0; j < C::JF; ++j) {
+    int base;
+    if constexpr (EPI == EPI_SILU) {
+      constexpr int HJ = C::JF / 2;
+      base = (j < HJ) ? wf * (C::TF / 2) + j * C::TILE : BF / 2 + wf * (C::TF / 2) + (j - HJ) * C::TILE;
+    } else {
+      base = wf * C::TF + j * C::TILE;
+    }
+    const int r = base + frow;
+    woff[j] = WBASE + r * CPR;
+    wkey[j] = swizzle<CPR>(r, 0);
+  }
+  acc_t acc[C::JF][C::IT];
+  u32x4 xf[2][C::IT][FC], wfr[2][C::JF][FC];
+
+  // ---- address sets: A = tile being multiplied, B = the workgroup's next tile --------
+  int pid_t, pid_f, expert;
+  int n_pid_t = 0, n_pid_f = 0, n_expert = 0;
+  int n_sid[XI * IW];  // sorted ids of the next tile's load rows (gather mode), fetched a tile ahead
+  unsigned xsrcA[XI * IW], wsrcA[WI * IW], xsrcB[XI * IW], wsrcB[WI * IW];
+  __amdgpu_buffer_rsrc_t xrsA, wrsA, xrsB, wrsB;
+#define FR_MAKE_SET(pt_, pf_, ex_, SIDOF, xsrc_, wsrc_, xrs_, wrs_)                                          \
+  {                                                                                                          \
+    const int64_t xrow0_ = a.top_k > 0 ? 0 : static_cast<int64_t>(pt_) * BT;                                 \
+    xrs_ = uniform_rsrc(X + xrow0_ * a.ldx);                                                                 \
+    wrs_ = uniform_rsrc(static_cast<const T*>(a.W) + static_cast<int64_t>(ex_) * a.w_expert_stride);         \
+    _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) {                                                 \
+      FR_SLOT_ROW(ih, rr, c)                                                                                 \
+      int64_t row_ = rr;                                                                                     \
+      if (a.top_k > 0) {                                                                                     \
+        const int sid_ = SIDOF;                                                                              \
+        row_ = sid_ < a.num_valid ? sid_ / a.top_k : 0;                                                      \
+      }                                                                                                      \
+      xsrc_[ih] = static_cast<unsigned>((row_ * a.ldx + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));    \
+    }                                                                                                        \
+    _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) {                                                 \
+      FR_SLOT_ROW(ih, rr, c)                                                                                 \
+      wsrc_[ih] = static_cast<unsigned>((static_cast<int64_t>(w_src_row(pf_, rr)) * a.ldw + k0 + c * EPC) * \
+                                        static_cast<int64_t>(sizeof(T)));                                    \
+    }                                                                                                        \
+  }
+  FR_COORDS(xbase + loc, pid_t, pid_f)
+  expert = a.expert_ids[pid_t];
+  FR_MAKE_SET(pid_t, pid_f, expert, a.sorted[pid_t * BT + rr], xsrcA, wsrcA, xrsA, wrsA)
+
+  // load q_ of an issuing wavefront (weight-tile loads first) of K tile tile_ into ring slot slot_
+#define FR_ISSUE_ONE(SET, tile_, slot_, q_)                                                                 \
+  {                                                                                                         \
+    const int vwi_ = wave_u + ((q_) % IW) * (NW / IW);                                                      \
+    if ((q_) < WI * IW) {                                                                                   \
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
+          wrs##SET, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vwi_) * (kWave * 16)), \
+          16, wsrc##SET[(q_) < WI * IW ? (q_) : 0], (tile_) * C::BKB, 0, 0);                                \
+    } else {                                                                                                \
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
+          xrs##SET, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WI * IW) / IW) * NW + vwi_) * (kWave * 16)), \
+          16, xsrc##SET[(q_) < WI * IW ? 0 : (q_) - WI * IW], (tile_) * C::BKB, 0, 0);                      \
+    }                                                                                                       \
+  }
+#define FR_READ_FRAGS(sl_, ks_, fb_)                                                    \
+  {                                                                                     \
+    const u32x4* xt = lds + (sl_) * C::XCH;                                             \
+    const u32x4* wtl = lds + (sl_) * C::WCH;                                            \
+    _Pragma("unroll") for (int c = 0; c < FC; ++c) {                                    \
+      const int kc = ((ks_) * C::KGROUPS + kgrp) * FC + c;                              \
+      _Pragma("unroll") for (int i = 0; i < C::IT; ++i)                                 \
+        xf[fb_][i][c] = xt[xoff[i] + (kc ^ xkey[i])];                                   \
+      _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                                 \
+        wfr[fb_][j][c] = wtl[woff[j] + (kc ^ wkey[j])];                                 \
+    }                                                                                   \
+  }
+  // One K-step: NM MFMAs; the fragments of the next step are read after the first half; the
+  // refill loads (ISS_: this wavefront issues, set SET) go out one at a time between the MFMAs.
+#define FR_KSTEP(fb_, READ_NEXT, ISS_, SET, tile_, slot_)                                     \
+  {                                                                                           \
+    _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                          \
+      const int j = m / C::IT, i = m % C::IT;                                                 \
+      if constexpr (C::TILE == 32) acc[j][i] = E::m32(wfr[fb_][j], xf[fb_][i], acc[j][i]);    \
+      else acc[j][i] = E::m16(wfr[fb_][j], xf[fb_][i], acc[j][i]);                            \
+      __builtin_amdgcn_sched_barrier(0);                                                      \
+      if (m == RD_AT) {                                                                       \
+        READ_NEXT;                                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                    \
+      }                                                                                       \
+      if (ISS_) {                                                                             \
+        _Pragma("unroll") for (int r = 0; r < NLI; ++r)                                       \
+          if (m == ((2 * r + 1) * NM) / (2 * NLI)) {                                          \
+            FR_ISSUE_ONE(SET, tile_, slot_, r);                                               \
+            __builtin_amdgcn_sched_barrier(0);                                                \
+          }                                                                                   \
+      }                                                                                       \
+    }                                                                                         \
+  }
+  // One K tile of the current output tile.  REFILL: 0 none (the data is the last this
+  // workgroup loads), else the slot of this K tile is refilled from set SET with K tile
+  // rtile_ after the barrier that publishes the next K tile; LAST: nothing follows this K
+  // tile at all (no barrier, no fragment read-ahead).
+#define FR_KTILE(ISS_, REFILL, SET, rtile_, LAST, VMC)                                         \
+  {                                                                                            \
+    const int sn = (sl + 1 == S) ? 0 : sl + 1;                                                 \
+    _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
+      if (ks + 1 < KS) {                                                                       \
+        FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, ks + 1, (ks + 1) & 1), false, A, 0, 0);             \
+      } else if (LAST) {                                                                       \
+        FR_KSTEP(ks & 1, {}, false, A, 0, 0);                                                  \
+      } else {                                                                                 \
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(VMC) : "memory");                  \
+        __builtin_amdgcn_s_barrier();                                                          \
+        FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, 0, 0), (ISS_) && (REFILL), SET, rtile_, sl);        \
+      }                                                                                        \
+    }                                                                                          \
+    sl = sn;                                                                                   \
+  }
+  // One output tile.  NEXT (compile time): the workgroup has another tile after this one, whose
+  // routing data is asked for at the start, turned into the address set B after two K tiles
+  // (straight-line code in between, so the wait for it is exact) and whose first S K tiles
+  // refill the ring during the last S K tiles of this one.
+#define FR_TILE(ISS_, NEXT)                                                                                \
+  {                                                                                                        \
+    if (NEXT) {                                                                                            \
+      FR_COORDS(xbase + loc + nper, n_pid_t, n_pid_f)                                                      \
+      n_expert = a.expert_ids[n_pid_t];                                                                    \
+      if (a.top_k > 0) {                                                                                   \
+        _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) {                                           \
+          FR_SLOT_ROW(ih, rr, c)                                                                           \
+          (void)c;                                                                                         \
+          n_sid[ih] = a.sorted[n_pid_t * BT + rr];                                                         \
+        }                                                                                                  \
+      }                                                                                                    \
+    }                                                                                                      \
+    _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                                                      \
+      _Pragma("unroll") for (int i = 0; i < C::IT; ++i)                                                    \
+        _Pragma("unroll") for (int r = 0; r < ACC_N; ++r) acc[j][i][r] = 0.f;                              \
+    /* vmcnt(0) once per tile: the previous tile's epilogue stores share the counter with the loads */     \
+    FR_KTILE(ISS_, true, A, S, false, 0)                                                                   \
+    FR_KTILE(ISS_, true, A, S + 1, false, (S - 2) * NLI)                                                   \
+    if (NEXT) FR_MAKE_SET(n_pid_t, n_pid_f, n_expert, n_sid[ih], xsrcB, wsrcB, xrsB, wrsB)                 \
+    __builtin_amdgcn_s_waitcnt(0xC07F); /* lgkmcnt(0): no scalar load pending inside the loops */          \
+    for (int kt = 2; kt < k_tiles - S; ++kt) FR_KTILE(ISS_, true, A, kt + S, false, (S - 2) * NLI)         \
+    if (NEXT) {                                                                                            \
+      for (int kt = 0; kt < S; ++kt) FR_KTILE(ISS_, true, B, kt, false, (S - 2) * NLI)                     \
+    } else {                                                                                               \
+      for (int kt = 0; kt < S - 1; ++kt) FR_KTILE(ISS_, false, A, 0, false, 0)                             \
+      FR_KTILE(ISS_, false, A, 0, true, 0)                                                                 \
+    }                                                                                                      \
+    gemm_epilogue<T, C, EPI>(a, acc, pid_t, pid_f, expert, split, wt, wf, frow, kgrp);                     \
+  }
+  // Whole pipeline for an issuing (ISS_ = true) or a non-issuing wavefront.
+#define FR_PERSIST(ISS_)                                                                                   \
+  {                                                                                                        \
+    _Pragma("unroll") for (int t = 0; t < S; ++t)                                                          \
+      if (ISS_) { _Pragma("unroll") for (int q = 0; q < NLI; ++q) FR_ISSUE_ONE(A, t, t, q); }               \
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((S - 1) * NLI) : "memory");                                   \
+    __builtin_amdgcn_s_barrier();                                                                          \
+    FR_READ_FRAGS(0, 0, 0);                                                                                \
+    int sl = 0;                                                                                            \
+    while (loc + nper < xcount) { /* a next tile exists: hand the ring over to it */                       \
+      FR_TILE(ISS_, true)                                                                                  \
+      pid_t = n_pid_t; pid_f = n_pid_f; expert = n_expert; xrsA = xrsB; wrsA = wrsB;                       \
+      _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) xsrcA[ih] = xsrcB[ih];                        \
+      _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) wsrcA[ih] = wsrcB[ih];                        \
+      loc += nper;                                                                                         \
+    }                                                                                                      \
+    FR_TILE(ISS_, false)                                                                                   \
+  }
+  if (IW == 1 || issuer) FR_PERSIST(true) else FR_PERSIST(false)
+#undef FR_PERSIST
+#undef FR_TILE
+#undef FR_KTILE
+#undef FR_KSTEP
+#undef FR_READ_FRAGS
+#undef FR_ISSUE_ONE
+#undef FR_MAKE_SET
+#undef FR_SLOT_ROW
+#undef FR_COORDS
+#endif
+}
+
+// Workgroups resident at once on the device (a multiple of 8, one share per XCD).
+template <typename T, typename C, int EPI>
+int persistent_grid(int* grid_out) {
+  static int cached = 0;
+  if (!cached) {
+    hipError_t e = hipSuccess;
+    if (C::LDS_BYTES > 65536)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_persistent_kernel<T, C, EPI>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    int dev = 0, cus = 0, per_cu = 0;
+    if (e == hipSuccess) e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e == hipSuccess)
+      e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, moe_gemm_persistent_kernel<T, C, EPI>, C::NT, C::LDS_BYTES);
+    if (e != hipSuccess) return fail(FR_E_LAUNCH, "persistent GEMM set-up (%d B LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
+    if (per_cu < 1 || cus < 8) return fail(FR_E_LAUNCH, "persistent GEMM: occupancy %d on %d CUs", per_cu, cus);
+    cached = cus * per_cu / 8 * 8;
+  }
+  *grid_out = cached;
+  return FR_OK;
+}
+
+// Launches the persistent form when every split has at least STAGES + 2 K tiles, else the plain one.
+template <typename T, typename C, int EPI>
+int launch_gemm_persistent(const GemmArgs& a, int splits, hipStream_t st) {
+  constexpr int BK = C::BKB / static_cast<int>(sizeof(T));
+  const int last_k = a.K - (splits - 1) * a.k_per_split;  // K range of the last split
+  if (a.k_per_split / BK < C::STAGES + 2 || last_k / BK < C::STAGES + 2) return launch_gemm<T, C, EPI>(a, splits, st);
+  const int64_t x_rows = a.top_k > 0 ? a.num_valid / a.top_k : C::BT;
+  const int64_t w_rows = EPI == EPI_SILU ? 2 * static_cast<int64_t>(a.N) : a.N;
+  const int64_t lim = int64_t(1) << 32, es = sizeof(T);
+  if (x_rows * a.ldx * es >= lim || w_rows * a.ldw * es >= lim)
+    return fail(FR_E_SHAPE, "token rows (%lld x %lld) or one expert's weights (%lld x %lld) span 4 GiB or more",
+                (long long)x_rows, (long long)a.ldx, (long long)w_rows, (long long)a.ldw);
+  int resident = 0;
+  const int rc = persistent_grid<T, C, EPI>(&resident);
+  if (rc != FR_OK) return rc;
+  const int64_t worst = static_cast<int64_t>(a.num_t_blocks) * a.num_f_tiles;
+  int64_t grid = resident / (splits > 1 ? splits : 1) / 8 * 8;  // the splits share the device
+  if (grid < 8) grid = 8;
+  if (grid > (worst + 7) / 8 * 8) grid = (worst + 7) / 8 * 8;
+  hipLaunchKernelGGL((moe_gemm_persistent_kernel<T, C, EPI>), dim3(static_cast<unsigned>(grid), splits), dim3(C::NT),
+                     C::LDS_BYTES, st, a);
+  return check_launch("moe_gemm_persistent_kernel");
+}
+
+}  // namespace fr

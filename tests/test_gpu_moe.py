@@ -164,6 +164,35 @@ def test_op_level_chain_matches_reference_layer_recipe(native, block):
     _assert_close(out, oracle.moe_experts(x, w1, w2, w, ids), dtype, "op chain")
 
 
+def test_block_256_several_tiles_per_workgroup(native):
+    """With more 256x256 tiles than resident workgroups the 2-byte kernel walks several
+    tiles per workgroup, the next tile's first loads issued during the current tile's last
+    K tiles: 27 token blocks x 16 feature tiles = 432 tiles for at most 256 workgroups,
+    so the grid mixes workgroups with one tile and with two."""
+    from fast_route_amd import fused_moe
+    from fast_route_amd.ops.fused_moe import invoke_fused_moe_kernel, moe_align_block_size
+    _say("block 256, several tiles per workgroup")
+    dtype = torch.bfloat16
+    M, H, Fd, E, k, block = 3000, 512, 2048, 4, 2, 256
+    x, logits, w1, w2 = _inputs(M, H, Fd, E, 33, dtype)
+    w, ids = oracle.gating_topk(logits, k)
+    xd, w1d, w2d, wd, idd = x.cuda(), w1.cuda(), w2.cuda(), w.cuda(), ids.cuda()
+    cfg = {"BLOCK_SIZE_M": block, "BLOCK_SIZE_N": 64, "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 8}
+    s, e, npost = moe_align_block_size(idd, block, E)
+    c1 = torch.empty((M, k, 2 * Fd), dtype=dtype, device="cuda")
+    invoke_fused_moe_kernel(xd, w1d, c1, wd, idd, s, e, npost, False, k, cfg)
+    _assert_close(c1.view(M * k, -1), oracle.grouped_gemm(x, w1, w, ids, False, k), dtype, "gemm1")
+    c2 = (torch.nn.functional.silu(c1[..., :Fd].float()) * c1[..., Fd:].float()).to(dtype).view(M * k, Fd)
+    c3 = torch.empty((M, k, H), dtype=dtype, device="cuda")
+    invoke_fused_moe_kernel(c2, w2d, c3, wd, idd, s, e, npost, True, 1, cfg)
+    torch.cuda.synchronize()
+    _assert_close(c3.float().sum(dim=1), oracle.moe_experts(x, w1, w2, w, ids), dtype, "op chain")
+    # the fused layer at the same size takes the same kernels through its own plan
+    out = fused_moe(xd, w1d, w2d, logits.cuda(), k, True)
+    torch.cuda.synchronize()
+    _assert_close(out, oracle.fused_moe(x, w1, w2, logits, k, True), dtype, "layer")
+
+
 def test_stable_and_vllm_route_layers(native):
     """Gate-matrix entry points of both reference layers."""
     from fast_route_amd.layers import stable_route, vllm_route
