@@ -75,6 +75,7 @@ class Layer:
         self.aws = torch.empty(max(self.aws_bytes, 256), dtype=torch.uint8, device=dev)
         self.act = torch.empty(p.sorted_len, self.F, dtype=torch.bfloat16, device=dev)
         self.partial = torch.empty(p.split_k * n * self.H, dtype=torch.float32, device=dev)
+        self.tail = torch.empty(p.tail_bytes, dtype=torch.uint8, device=dev) if p.tail_bytes else None
         if fp8:
             self.xq = torch.empty(M, self.H, dtype=torch.uint8, device=dev)
             self.xs = torch.empty(M, dtype=torch.float32, device=dev)
@@ -122,12 +123,14 @@ class Layer:
             return
         N.check(lib.fr_moe_gateup_silu(self.x.data_ptr(), self.w1.data_ptr(), self.sorted.data_ptr(), self.eids.data_ptr(),
                                        self.npost.data_ptr(), self.M, self.H, self.F, self.E, self.topk, p.block, N.FR_BF16,
-                                       self.act.data_ptr(), self.stream))
+                                       self.act.data_ptr(), self.tail.data_ptr() if self.tail is not None else None,
+                                       self.stream))
         rec(3)
         N.check(lib.fr_moe_down_combine(self.act.data_ptr(), self.w2.data_ptr(), self.tw.data_ptr(), self.sorted.data_ptr(),
                                         self.eids.data_ptr(), self.npost.data_ptr(), self.M, self.H, self.F, self.E,
                                         self.topk, p.block, p.split_k, N.FR_BF16, self.partial.data_ptr(),
-                                        self.out.data_ptr(), self.stream))
+                                        self.out.data_ptr(), self.tail.data_ptr() if self.tail is not None else None,
+                                        self.stream))
         rec(4)
 
     def active_experts(self):

@@ -15,7 +15,7 @@ _SHAPE_ERRORS = (-1, -2, -3, -4, -5)  # argument errors -> AssertionError like t
 
 class FrMoePlan(ctypes.Structure):
     _fields_ = [("block", c_int32), ("split_k", c_int32), ("sorted_len", c_int64),
-                ("workspace_bytes", c_int64)]
+                ("workspace_bytes", c_int64), ("tail_bytes", c_int64)]
 
 
 # name -> (restype, argtypes); must list every symbol the header declares
@@ -30,9 +30,9 @@ SIGNATURES = {
                                     c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fr_moe_get_plan": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, c_int, ctypes.POINTER(FrMoePlan)]),
     "fr_moe_gateup_silu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
-                                   c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+                                   c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "fr_moe_down_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
-                                    c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+                                    c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "fr_fused_experts": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                  c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_void_p]),
     "fr_quant_e4m3_rows": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),

@@ -14,6 +14,11 @@ int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
 
 // per-row e4m3 quantisation; rows_dev (optional, device) bounds the rows actually touched
+// Bytes of the scratch with which a grouped GEMM of this routing block, operand type, K (elements)
+// and output feature count N can split the tiles of its last round along K; 0 if it cannot.
+// gateup: N counts the activated features (the weight has 2N rows).
+int64_t tail_scratch_bytes(int block, int dtype, int64_t K, int64_t N, bool gateup);
+
 int quant_rows(const void* x, int dtype, int64_t rows, const int32_t* rows_dev, int64_t K, int64_t ldx, void* q_out,
                float* scale_out, hipStream_t st);
 

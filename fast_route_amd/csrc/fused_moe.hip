@@ -18,6 +18,7 @@ struct Carve {
   int64_t align_ws_bytes;
   void* act;
   float* partial;
+  float* tail;       // scratch for splitting the last round of 256-row tiles, or nullptr
   void* xq;          // fp8 layer only
   float* x_scale;
   void* actq;
@@ -43,6 +44,7 @@ Carve carve(void* base, int64_t M, int64_t H, int64_t F, int E, int topk, int dt
   c.align_ws = take(c.align_ws_bytes);
   c.act = take(p.sorted_len * F * act_elem_size(dtype));
   c.partial = reinterpret_cast<float*>(take(static_cast<int64_t>(p.split_k) * n * H * 4));
+  c.tail = p.tail_bytes > 0 ? reinterpret_cast<float*>(take(p.tail_bytes)) : nullptr;
   c.xq = nullptr; c.x_scale = nullptr; c.actq = nullptr; c.act_scale = nullptr;
   if (dtype == FR_FP8_E4M3) {
     c.xq = take(M * H);
@@ -88,8 +90,13 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   const int64_t blocks = n <= E ? n : (block >= 128 ? ceil_div(n, block) + E / 2 : E);
   const int64_t tiles = blocks * ceil_div(H, bf);
   const int bk_elems = dtype == FR_FP8_E4M3 ? (block <= 32 ? 256 : 128) : (block == 16 ? 128 : 64);
+  // 256-row tiles of 2-byte operands with a long K balance their last round themselves (its
+  // tiles are cut along K over the idle workgroups); both GEMMs share the scratch for that.
+  const int64_t tail_up = tail_scratch_bytes(block, dtype, H, F, true), tail_down = tail_scratch_bytes(block, dtype, F, H, false);
   int split = 1;
-  if (block >= 128) {
+  if (tail_down > 0) {
+    split = 1;
+  } else if (block >= 128) {
     // one workgroup per CU: pick the split whose grid fills whole rounds of 256 CUs best,
     // charging 7 % per extra fp32 partial slice (its write + re-read in the combine)
     double best = -1.0;
@@ -106,6 +113,7 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   plan->block = block;
   plan->split_k = split;
   plan->sorted_len = n + static_cast<int64_t>(E) * (block - 1);
+  plan->tail_bytes = tail_up > tail_down ? tail_up : tail_down;
   plan->workspace_bytes = carve(nullptr, M, H, F, E, topk, dtype, *plan).total;
   return FR_OK;
 }
@@ -139,9 +147,9 @@ extern "C" int fr_fused_experts(const void* x, const void* w1, const void* w2, c
   Carve c = carve(workspace, M, H, F, E, topk, dtype, p);
   rc = fr_moe_align(topk_ids, FR_I32, M * topk, E, p.block, c.sorted, c.expert_ids, c.npost, c.align_ws, c.align_ws_bytes, stream);
   if (rc != FR_OK) return rc;
-  rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, stream);
+  rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, c.tail, stream);
   if (rc != FR_OK) return rc;
-  return fr_moe_down_combine(c.act, w2, topk_weights, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, p.split_k, dtype, c.partial, out, stream);
+  return fr_moe_down_combine(c.act, w2, topk_weights, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, p.split_k, dtype, c.partial, out, c.tail, stream);
 }
 
 extern "C" int fr_fused_moe(const void* x, const void* w1, const void* w2, const void* logits, int logits_dtype,
@@ -157,9 +165,9 @@ extern "C" int fr_fused_moe(const void* x, const void* w1, const void* w2, const
   Carve c = carve(workspace, M, H, F, E, topk, dtype, p);
   rc = route_and_align(logits, logits_dtype, M, E, topk, renormalize, p.block, c, stream);
   if (rc != FR_OK) return rc;
-  rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, stream);
+  rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, c.tail, stream);
   if (rc != FR_OK) return rc;
-  return fr_moe_down_combine(c.act, w2, c.topk_w, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, p.split_k, dtype, c.partial, out, stream);
+  return fr_moe_down_combine(c.act, w2, c.topk_w, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, p.split_k, dtype, c.partial, out, c.tail, stream);
 }
 
 extern "C" int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, const float* w1_scale, const void* w2q,

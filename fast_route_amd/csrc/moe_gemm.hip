@@ -128,9 +128,18 @@ int usable_splits(int split_k, int64_t K, int bk) {
   return splits;
 }
 
+int64_t tail_scratch_bytes(int block, int dtype, int64_t K, int64_t N, bool gateup) {
+  typedef Tiles<bf16_t>::T256 C;  // the one tile that runs persistently (2-byte operands only)
+  if (block != 256 || (dtype != FR_BF16 && dtype != FR_F16)) return 0;
+  const int64_t bk = C::BKB / 2, cols = gateup ? C::BF / 2 : C::BF;
+  if (K / bk < kTailMinTiles || N % cols != 0) return 0;
+  return static_cast<int64_t>(kTailUnits) * C::BT * C::BF * 4;
+}
+
 int gateup_impl(const void* x, const float* x_scale, const void* w1, const float* w1_scale,
                 const int32_t* sorted, const int32_t* expert_ids, const int32_t* npost, int64_t M, int64_t H,
-                int64_t F, int E, int topk, int block, int dtype, void* act, hipStream_t st, const char* who) {
+                int64_t F, int E, int topk, int block, int dtype, void* act, float* tail_ws, hipStream_t st,
+                const char* who) {
   if (M == 0) return FR_OK;
   FR_REQUIRE(x && w1 && act && sorted && expert_ids && npost, FR_E_NULL, "%s: null pointer", who);
   FR_REQUIRE(valid_block(block), FR_E_SHAPE, "%s: block=%d not in {16,32,64,128,256}", who, block);
@@ -144,13 +153,14 @@ int gateup_impl(const void* x, const float* x_scale, const void* w1, const float
   a.sorted = sorted; a.expert_ids = expert_ids; a.npost = npost;
   a.x_scale = x_scale; a.w_scale = w1_scale; a.w_rows = static_cast<int>(2 * F);
   a.num_valid = (int)n; a.top_k = topk; a.N = (int)F; a.K = (int)H;
+  a.tail_ws = tail_ws;
   return dispatch_dtype<EPI_SILU>(a, dtype, block, 1, sorted_len / block * block, st);
 }
 
 int down_impl(const void* act, const float* act_scale, const void* w2, const float* w2_scale,
               const float* topk_weights, const int32_t* sorted, const int32_t* expert_ids, const int32_t* npost,
               int64_t M, int64_t H, int64_t F, int E, int topk, int block, int split_k, int dtype, int out_dtype,
-              float* partial, void* out, hipStream_t st, const char* who) {
+              float* partial, void* out, float* tail_ws, hipStream_t st, const char* who) {
   if (M == 0) return FR_OK;
   FR_REQUIRE(act && w2 && topk_weights && partial && out && sorted && expert_ids && npost, FR_E_NULL, "%s: null pointer", who);
   FR_REQUIRE(valid_block(block), FR_E_SHAPE, "%s: block=%d not in {16,32,64,128,256}", who, block);
@@ -168,6 +178,7 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
   a.x_scale = act_scale; a.w_scale = w2_scale; a.w_rows = static_cast<int>(H);
   a.topk_w = topk_weights; a.num_valid = (int)n; a.top_k = 0; a.N = (int)H; a.K = (int)F;
   a.mul_weight = 1;
+  a.tail_ws = tail_ws;
   int rc = dispatch_dtype<EPI_DOWN>(a, dtype, block, splits, sorted_len / block * block, st);
   if (rc != FR_OK) return rc;
   return launch_combine(partial, n * H, splits, topk, M, (int)H, out_dtype, out, st);
@@ -204,10 +215,10 @@ extern "C" int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, vo
 extern "C" int fr_moe_gateup_silu(const void* x, const void* w1, const int32_t* sorted_token_ids,
                                   const int32_t* expert_ids, const int32_t* num_tokens_post_pad,
                                   int64_t M, int64_t H, int64_t F, int E, int topk, int block, int dtype,
-                                  void* act, void* stream) {
+                                  void* act, void* tail_ws, void* stream) {
   FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "fr_moe_gateup_silu: dtype %d not in {f16, bf16}", dtype);
   return gateup_impl(x, nullptr, w1, nullptr, sorted_token_ids, expert_ids, num_tokens_post_pad, M, H, F, E, topk,
-                     block, dtype, act, static_cast<hipStream_t>(stream), "fr_moe_gateup_silu");
+                     block, dtype, act, static_cast<float*>(tail_ws), static_cast<hipStream_t>(stream), "fr_moe_gateup_silu");
 }
 
 extern "C" int fr_moe_gateup_silu_fp8(const void* xq, const float* x_scale, const void* w1q, const float* w1_scale,
@@ -216,17 +227,18 @@ extern "C" int fr_moe_gateup_silu_fp8(const void* xq, const float* x_scale, cons
                                       int topk, int block, void* act_bf16, void* stream) {
   FR_REQUIRE(x_scale && w1_scale, FR_E_NULL, "fr_moe_gateup_silu_fp8: null scale pointer");
   return gateup_impl(xq, x_scale, w1q, w1_scale, sorted_token_ids, expert_ids, num_tokens_post_pad, M, H, F, E, topk,
-                     block, FR_FP8_E4M3, act_bf16, static_cast<hipStream_t>(stream), "fr_moe_gateup_silu_fp8");
+                     block, FR_FP8_E4M3, act_bf16, nullptr, static_cast<hipStream_t>(stream), "fr_moe_gateup_silu_fp8");
 }
 
 extern "C" int fr_moe_down_combine(const void* act, const void* w2, const float* topk_weights,
                                    const int32_t* sorted_token_ids, const int32_t* expert_ids,
                                    const int32_t* num_tokens_post_pad, int64_t M, int64_t H, int64_t F,
                                    int E, int topk, int block, int split_k, int dtype, float* partial,
-                                   void* out, void* stream) {
+                                   void* out, void* tail_ws, void* stream) {
   FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "fr_moe_down_combine: dtype %d not in {f16, bf16}", dtype);
   return down_impl(act, nullptr, w2, nullptr, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, M, H, F,
-                   E, topk, block, split_k, dtype, dtype, partial, out, static_cast<hipStream_t>(stream), "fr_moe_down_combine");
+                   E, topk, block, split_k, dtype, dtype, partial, out, static_cast<float*>(tail_ws),
+                   static_cast<hipStream_t>(stream), "fr_moe_down_combine");
 }
 
 extern "C" int fr_moe_down_combine_fp8(const void* actq, const float* act_scale, const void* w2q, const float* w2_scale,
@@ -236,6 +248,6 @@ extern "C" int fr_moe_down_combine_fp8(const void* actq, const float* act_scale,
                                        float* partial, void* out, void* stream) {
   FR_REQUIRE(act_scale && w2_scale, FR_E_NULL, "fr_moe_down_combine_fp8: null scale pointer");
   return down_impl(actq, act_scale, w2q, w2_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, M,
-                   H, F, E, topk, block, split_k, FR_FP8_E4M3, out_dtype, partial, out, static_cast<hipStream_t>(stream),
-                   "fr_moe_down_combine_fp8");
+                   H, F, E, topk, block, split_k, FR_FP8_E4M3, out_dtype, partial, out, nullptr,
+                   static_cast<hipStream_t>(stream), "fr_moe_down_combine_fp8");
 }

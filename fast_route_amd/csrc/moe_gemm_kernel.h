@@ -47,6 +47,7 @@ struct GemmArgs {
   int num_f_tiles;
   int group_t;
   int mul_weight;
+  float* tail_ws;       // persistent form only: slice buffers for splitting the last round of tiles along K, or nullptr
 };
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));

@@ -9,10 +9,81 @@
 //
 // Same tile shapes, LDS layout, swizzle, fragment double buffering, barrier placement and
 // epilogues as moe_gemm_kernel (STAGES >= 2, refill in one group); see there.
+//
+// Tail split.  The tiles of an XCD rarely fill whole rounds of its workgroups: with 70 tiles
+// for 32 workgroups the third round keeps 6 of them busy.  Given scratch (GemmArgs::tail_ws)
+// the tiles of that last round are split along K into as many slices as there are idle
+// workgroups per tile (at most kTailMaxSplit, each at least kTailMinSlice K tiles long); a
+// slice is one more work unit of its workgroup, its fp32 accumulators go to the scratch as
+// they are, and tail_fixup_kernel sums the slices of a tile in slice order and applies the
+// epilogue.  Nothing waits on another workgroup and the result does not depend on timing.
 #pragma once
 #include "moe_gemm_kernel.h"
 
 namespace fr {
+
+constexpr int kTailMaxSplit = 8;    // K slices per tile of the last round, at most
+constexpr int kTailMinSlice = 8;    // K tiles per slice, at least
+constexpr int kTailMinTiles = 32;   // K tiles per output tile below which the split is not worth its fix-up launch
+constexpr int kTailUnits = 256;     // workgroups (= slice buffers in the scratch), at most
+
+// Tiles of one XCD: a contiguous range of the real tile count, `rounds` whole rounds of the
+// XCD's `nper` workgroups and `rest` tiles after them, each cut into `slices` K slices.
+struct XcdSchedule {
+  int base, count, rounds, rest, slices;
+};
+__device__ __forceinline__ XcdSchedule xcd_schedule(int total, int nper, int xcd, int k_tiles, bool split_tail) {
+  XcdSchedule s;
+  const int per = total >> 3, rem = total & 7;
+  s.base = xcd * per + (xcd < rem ? xcd : rem);
+  s.count = per + (xcd < rem ? 1 : 0);
+  s.rounds = s.count / nper;
+  s.rest = s.count - s.rounds * nper;
+  s.slices = 1;
+  if (split_tail && s.rest > 0) {
+    // Worth it when the time saved, about (0.7 - 1/slices) of a tile's K loop, exceeds the
+    // fix-up's: one fp32 tile written and read back per slice plus a launch, in units of
+    // about a twelfth of a K tile's time (measured: 10 tiles in 3 slices of 21 K tiles each
+    // break even or gain, 6 tiles in 5 slices of 45 gain a fifth of the kernel's time).
+    const int sl = min(min(nper / s.rest, k_tiles / kTailMinSlice), kTailMaxSplit);
+    if (sl >= 2 && k_tiles * (7 * sl - 10) >= 3 * sl * (s.rest * sl + 10)) s.slices = sl;
+  }
+  return s;
+}
+// Walk order of the tiles: groups of group_t token blocks x all feature tiles.
+__device__ __forceinline__ void tile_coords(const GemmArgs& a, int nt, int lin, int& pid_t, int& pid_f) {
+  const int in_group = a.group_t * a.num_f_tiles;
+  const int first = (lin / in_group) * a.group_t;
+  const int gsz = min(nt - first, a.group_t);
+  pid_t = first + (lin % in_group) % gsz;
+  pid_f = (lin % in_group) / gsz;
+}
+// Tile column of accumulator tile j of feature wavefront wf (= row of the weight tile in LDS).
+template <typename C, int EPI>
+__device__ __forceinline__ int acc_tile_col(int wf, int j) {
+  if constexpr (EPI == EPI_SILU) {
+    constexpr int HJ = C::JF / 2;  // first half of the wave's tiles: gate, second: up
+    return (j < HJ) ? wf * (C::TF / 2) + j * C::TILE : C::BF / 2 + wf * (C::TF / 2) + (j - HJ) * C::TILE;
+  } else {
+    return wf * C::TF + j * C::TILE;
+  }
+}
+// fp32 accumulators of one K slice, as they are, to the slice's [BT][BF] buffer
+template <typename C, int EPI, typename AccT>
+__device__ __forceinline__ void tail_store(float* tile, AccT (&acc)[C::JF][C::IT], int wt, int wf, int frow, int kgrp) {
+  constexpr int GROUPS = ((C::TILE == 32) ? 16 : 4) / 4;
+#pragma unroll
+  for (int i = 0; i < C::IT; ++i) {
+    float* row = tile + (wt * C::TT + i * C::TILE + frow) * C::BF;
+#pragma unroll
+    for (int j = 0; j < C::JF; ++j)
+#pragma unroll
+      for (int g = 0; g < GROUPS; ++g) {
+        const f32x4 o = {acc[j][i][g * 4 + 0], acc[j][i][g * 4 + 1], acc[j][i][g * 4 + 2], acc[j][i][g * 4 + 3]};
+        *reinterpret_cast<f32x4*>(row + acc_tile_col<C, EPI>(wf, j) + g * 8 + kgrp * 4) = o;
+      }
+  }
+}
 
 template <typename T, typename C, int EPI>
 __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(const GemmArgs a) {
@@ -41,31 +112,40 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   // The real tile count is dealt to the 8 XCDs (workgroup id mod 8) in contiguous ranges; the
   // workgroups of one XCD take the tiles of its range round robin, so at any moment they work on
   // consecutive tiles (group_t token blocks x consecutive feature tiles: shared in that XCD's L2).
+  // Work unit j of a workgroup: tile j of its round-robin walk over all K tiles, or, after the
+  // whole rounds, one K slice of a tile of the last round.
   const int npost = a.npost[0];
   const int nt = min(npost / BT, a.num_t_blocks);
   const int total = nt * a.num_f_tiles;
-  const int xcd = blockIdx.x & 7, nper = gridDim.x >> 3;
-  const int per = total >> 3, rem = total & 7;
-  const int xbase = xcd * per + (xcd < rem ? xcd : rem), xcount = per + (xcd < rem ? 1 : 0);
-  int loc = blockIdx.x >> 3;
-  if (loc >= xcount) return;
-  const int in_group = a.group_t * a.num_f_tiles;
+  const int xcd = blockIdx.x & 7, nper = gridDim.x >> 3, loc = blockIdx.x >> 3;
   const int split = blockIdx.y;
+  const int k0 = split * a.k_per_split;
+  const int k_all = min(a.k_per_split, a.K - k0) / BK;  // K tiles of a whole unit, >= S + 2 (checked by the launcher)
+  const XcdSchedule xs = xcd_schedule(total, nper, xcd, k_all, a.tail_ws != nullptr);
+  const int n_units = xs.rounds + (loc < xs.rest * xs.slices ? 1 : 0);
+  if (n_units == 0) return;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wt = wave / C::WF, wf = wave % C::WF;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const bool issuer = wave_u < NW / IW;
   const T* X = static_cast<const T*>(a.X);
-  const int k0 = split * a.k_per_split;
-  const int k_tiles = min(a.k_per_split, a.K - k0) / BK;  // >= S + 2 (checked by the launcher)
 
-#define FR_COORDS(lin_, pt_, pf_)                                  \
-  {                                                                \
-    const int gid_ = (lin_) / in_group, first_ = gid_ * a.group_t; \
-    const int gsz_ = min(nt - first_, a.group_t);                  \
-    pt_ = first_ + ((lin_) % in_group) % gsz_;                     \
-    pf_ = ((lin_) % in_group) / gsz_;                              \
+  // unit j_ -> tile coordinates, first K tile kb_ and K tile count kn_, slice buffer tu_ (-1: a whole tile)
+#define FR_UNIT(j_, pt_, pf_, kb_, kn_, tu_)                                                   \
+  {                                                                                            \
+    int lin_;                                                                                  \
+    if ((j_) < xs.rounds) {                                                                    \
+      lin_ = xs.base + (j_) * nper + loc;                                                      \
+      kb_ = 0; kn_ = k_all; tu_ = -1;                                                          \
+    } else {                                                                                   \
+      const int t_ = loc % xs.rest, s_ = loc / xs.rest;                                        \
+      lin_ = xs.base + xs.rounds * nper + t_;                                                  \
+      kb_ = s_ * k_all / xs.slices;                                                            \
+      kn_ = (s_ + 1) * k_all / xs.slices - kb_;                                                \
+      tu_ = xs.slices > 1 ? s_ * xs.rest + t_ : -1;                                            \
+    }                                                                                          \
+    tile_coords(a, nt, lin_, pt_, pf_);                                                        \
   }
   // rows of the load slots this wavefront issues: load index ih -> tile row
 #define FR_SLOT_ROW(ih_, rr_, c_)                                                  \
@@ -93,13 +173,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   }
 #pragma unroll
   for (int j = 0; j < C::JF; ++j) {
-    int base;
-    if constexpr (EPI == EPI_SILU) {
-      constexpr int HJ = C::JF / 2;
-      base = (j < HJ) ? wf * (C::TF / 2) + j * C::TILE : BF / 2 + wf * (C::TF / 2) + (j - HJ) * C::TILE;
-    } else {
-      base = wf * C::TF + j * C::TILE;
-    }
+    const int base = acc_tile_col<C, EPI>(wf, j);
     const int r = base + frow;
     woff[j] = WBASE + r * CPR;
     wkey[j] = swizzle<CPR>(r, 0);
@@ -108,14 +182,15 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   u32x4 xf[2][C::IT][FC], wfr[2][C::JF][FC];
 
   // ---- address sets: A = tile being multiplied, B = the workgroup's next tile --------
-  int pid_t, pid_f, expert;
-  int n_pid_t = 0, n_pid_f = 0, n_expert = 0;
+  int pid_t, pid_f, expert, kb, kn, tu;  // current unit: tile, first K tile and K tile count, slice buffer
+  int n_pid_t = 0, n_pid_f = 0, n_expert = 0, n_kb = 0, n_kn = 0, n_tu = -1;
   int n_sid[XI * IW];  // sorted ids of the next tile's load rows (gather mode), fetched a tile ahead
   unsigned xsrcA[XI * IW], wsrcA[WI * IW], xsrcB[XI * IW], wsrcB[WI * IW];
   __amdgpu_buffer_rsrc_t xrsA, wrsA, xrsB, wrsB;
-#define FR_MAKE_SET(pt_, pf_, ex_, SIDOF, xsrc_, wsrc_, xrs_, wrs_)                                          \
+#define FR_MAKE_SET(pt_, pf_, ex_, kb_, SIDOF, xsrc_, wsrc_, xrs_, wrs_)                                     \
   {                                                                                                          \
     const int64_t xrow0_ = a.top_k > 0 ? 0 : static_cast<int64_t>(pt_) * BT;                                 \
+    const int64_t kfirst_ = k0 + static_cast<int64_t>(kb_) * BK;                                             \
     xrs_ = uniform_rsrc(X + xrow0_ * a.ldx);                                                                 \
     wrs_ = uniform_rsrc(static_cast<const T*>(a.W) + static_cast<int64_t>(ex_) * a.w_expert_stride);         \
     _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) {                                                 \
@@ -125,17 +200,17 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
         const int sid_ = SIDOF;                                                                              \
         row_ = sid_ < a.num_valid ? sid_ / a.top_k : 0;                                                      \
       }                                                                                                      \
-      xsrc_[ih] = static_cast<unsigned>((row_ * a.ldx + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));    \
+      xsrc_[ih] = static_cast<unsigned>((row_ * a.ldx + kfirst_ + c * EPC) * static_cast<int64_t>(sizeof(T))); \
     }                                                                                                        \
     _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) {                                                 \
       FR_SLOT_ROW(ih, rr, c)                                                                                 \
-      wsrc_[ih] = static_cast<unsigned>((static_cast<int64_t>(w_src_row(pf_, rr)) * a.ldw + k0 + c * EPC) * \
+      wsrc_[ih] = static_cast<unsigned>((static_cast<int64_t>(w_src_row(pf_, rr)) * a.ldw + kfirst_ + c * EPC) * \
                                         static_cast<int64_t>(sizeof(T)));                                    \
     }                                                                                                        \
   }
-  FR_COORDS(xbase + loc, pid_t, pid_f)
+  FR_UNIT(0, pid_t, pid_f, kb, kn, tu)
   expert = a.expert_ids[pid_t];
-  FR_MAKE_SET(pid_t, pid_f, expert, a.sorted[pid_t * BT + rr], xsrcA, wsrcA, xrsA, wrsA)
+  FR_MAKE_SET(pid_t, pid_f, expert, kb, a.sorted[pid_t * BT + rr], xsrcA, wsrcA, xrsA, wrsA)
 
   // load q_ of an issuing wavefront (weight-tile loads first) of K tile tile_ into ring slot slot_
 #define FR_ISSUE_ONE(SET, tile_, slot_, q_)                                                                 \
@@ -212,7 +287,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #define FR_TILE(ISS_, NEXT)                                                                                \
   {                                                                                                        \
     if (NEXT) {                                                                                            \
-      FR_COORDS(xbase + loc + nper, n_pid_t, n_pid_f)                                                      \
+      FR_UNIT(unit + 1, n_pid_t, n_pid_f, n_kb, n_kn, n_tu)                                                \
       n_expert = a.expert_ids[n_pid_t];                                                                    \
       if (a.top_k > 0) {                                                                                   \
         _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) {                                           \
@@ -228,16 +303,17 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     /* vmcnt(0) once per tile: the previous tile's epilogue stores share the counter with the loads */     \
     FR_KTILE(ISS_, true, A, S, false, 0)                                                                   \
     FR_KTILE(ISS_, true, A, S + 1, false, (S - 2) * NLI)                                                   \
-    if (NEXT) FR_MAKE_SET(n_pid_t, n_pid_f, n_expert, n_sid[ih], xsrcB, wsrcB, xrsB, wrsB)                 \
+    if (NEXT) FR_MAKE_SET(n_pid_t, n_pid_f, n_expert, n_kb, n_sid[ih], xsrcB, wsrcB, xrsB, wrsB)           \
     __builtin_amdgcn_s_waitcnt(0xC07F); /* lgkmcnt(0): no scalar load pending inside the loops */          \
-    for (int kt = 2; kt < k_tiles - S; ++kt) FR_KTILE(ISS_, true, A, kt + S, false, (S - 2) * NLI)         \
+    for (int kt = 2; kt < kn - S; ++kt) FR_KTILE(ISS_, true, A, kt + S, false, (S - 2) * NLI)              \
     if (NEXT) {                                                                                            \
       for (int kt = 0; kt < S; ++kt) FR_KTILE(ISS_, true, B, kt, false, (S - 2) * NLI)                     \
     } else {                                                                                               \
       for (int kt = 0; kt < S - 1; ++kt) FR_KTILE(ISS_, false, A, 0, false, 0)                             \
       FR_KTILE(ISS_, false, A, 0, true, 0)                                                                 \
     }                                                                                                      \
-    gemm_epilogue<T, C, EPI>(a, acc, pid_t, pid_f, expert, split, wt, wf, frow, kgrp);                     \
+    if (tu < 0) gemm_epilogue<T, C, EPI>(a, acc, pid_t, pid_f, expert, split, wt, wf, frow, kgrp);         \
+    else tail_store<C, EPI>(a.tail_ws + static_cast<int64_t>(xcd * nper + tu) * (BT * BF), acc, wt, wf, frow, kgrp); \
   }
   // Whole pipeline for an issuing (ISS_ = true) or a non-issuing wavefront.
 #define FR_PERSIST(ISS_)                                                                                   \
@@ -248,12 +324,13 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     __builtin_amdgcn_s_barrier();                                                                          \
     FR_READ_FRAGS(0, 0, 0);                                                                                \
     int sl = 0;                                                                                            \
-    while (loc + nper < xcount) { /* a next tile exists: hand the ring over to it */                       \
+    int unit = 0;                                                                                          \
+    for (; unit + 1 < n_units; ++unit) { /* a next unit exists: hand the ring over to it */                \
       FR_TILE(ISS_, true)                                                                                  \
       pid_t = n_pid_t; pid_f = n_pid_f; expert = n_expert; xrsA = xrsB; wrsA = wrsB;                       \
+      kb = n_kb; kn = n_kn; tu = n_tu;                                                                     \
       _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) xsrcA[ih] = xsrcB[ih];                        \
       _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) wsrcA[ih] = wsrcB[ih];                        \
-      loc += nper;                                                                                         \
     }                                                                                                      \
     FR_TILE(ISS_, false)                                                                                   \
   }
@@ -266,8 +343,64 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #undef FR_ISSUE_ONE
 #undef FR_MAKE_SET
 #undef FR_SLOT_ROW
-#undef FR_COORDS
+#undef FR_UNIT
 #endif
+}
+
+// Sums the K slices of the tiles of each XCD's last round in slice order and applies the
+// epilogue the GEMM would have applied: routed weight and scatter to the pair's row of the
+// fp32 partial buffer (EPI_DOWN), or silu(gate)*up to the slot's row of act (EPI_SILU).
+// Grid: 8 XCDs x nper/2 tiles (a split tail has at most that many) x BT/32 row groups; blocks
+// without a split tile leave at once.  nper = workgroups per XCD of the GEMM launch.
+constexpr int kFixupRows = 32;
+template <typename T, typename C, int EPI>
+__global__ __launch_bounds__(256) void tail_fixup_kernel(const GemmArgs a, int nper) {
+  typedef Elem<T> E;
+  typedef typename E::out_t out_t;
+  typedef typename E::out4 out4;
+  static_assert(EPI == EPI_SILU || EPI == EPI_DOWN, "fix-up of the fused epilogues only");
+  constexpr int BT = C::BT, BF = C::BF, BK = C::BKB / static_cast<int>(sizeof(T));
+  constexpr int COLS = (EPI == EPI_SILU) ? BF / 2 : BF;  // output columns of a tile
+  constexpr int CG = COLS / 4, RPP = 256 / CG;           // 4-column groups per row, rows per pass
+  static_assert(256 % CG == 0 && kFixupRows % RPP == 0 && BT % kFixupRows == 0, "fix-up thread map");
+  constexpr int BPT = BT / kFixupRows;
+  const int half = nper / 2;
+  const int xcd = blockIdx.x / (half * BPT), t = (blockIdx.x / BPT) % half, rb = blockIdx.x % BPT;
+  const int nt = min(a.npost[0] / BT, a.num_t_blocks);
+  const XcdSchedule xs = xcd_schedule(nt * a.num_f_tiles, nper, xcd, a.K / BK, true);
+  if (xs.slices < 2 || t >= xs.rest) return;
+  int pid_t, pid_f;
+  tile_coords(a, nt, xs.base + xs.rounds * nper + t, pid_t, pid_f);
+  const float* first = a.tail_ws + static_cast<int64_t>(xcd * nper + t) * (BT * BF);
+  const int64_t slice_stride = static_cast<int64_t>(xs.rest) * (BT * BF);
+  const int cg = threadIdx.x % CG;
+#pragma unroll
+  for (int p = 0; p < kFixupRows / RPP; ++p) {
+    const int row = rb * kFixupRows + p * RPP + threadIdx.x / CG;
+    const int slot = pid_t * BT + row;
+    const float* src = first + row * BF + cg * 4;
+    if constexpr (EPI == EPI_DOWN) {
+      const int sid = a.sorted[slot];
+      if (sid >= a.num_valid) continue;
+      f32x4 sum = *reinterpret_cast<const f32x4*>(src);
+      for (int s = 1; s < xs.slices; ++s) sum += *reinterpret_cast<const f32x4*>(src + s * slice_stride);
+      const float rw = a.mul_weight ? a.topk_w[sid] : 1.f;
+      float* orow = static_cast<float*>(a.out) + static_cast<int64_t>(sid) * a.ldo + pid_f * BF + cg * 4;
+      const f32x4 o = {sum[0] * rw, sum[1] * rw, sum[2] * rw, sum[3] * rw};
+      *reinterpret_cast<f32x4*>(orow) = o;
+    } else {
+      f32x4 g = *reinterpret_cast<const f32x4*>(src), u = *reinterpret_cast<const f32x4*>(src + BF / 2);
+      for (int s = 1; s < xs.slices; ++s) {
+        g += *reinterpret_cast<const f32x4*>(src + s * slice_stride);
+        u += *reinterpret_cast<const f32x4*>(src + s * slice_stride + BF / 2);
+      }
+      out4 o;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[r] = static_cast<out_t>(silu(g[r]) * u[r]);
+      out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(slot) * a.ldo + pid_f * (BF / 2) + cg * 4;
+      *reinterpret_cast<out4*>(orow) = o;
+    }
+  }
 }
 
 // Workgroups resident at once on the device (a multiple of 8, one share per XCD).
@@ -293,11 +426,16 @@ int persistent_grid(int* grid_out) {
 }
 
 // Launches the persistent form when every split has at least STAGES + 2 K tiles, else the plain one.
+// a.tail_ws (kTailUnits buffers of BT x BF floats, or nullptr) enables the split of the last round.
 template <typename T, typename C, int EPI>
-int launch_gemm_persistent(const GemmArgs& a, int splits, hipStream_t st) {
+int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
+  GemmArgs a = a_in;
   constexpr int BK = C::BKB / static_cast<int>(sizeof(T));
   const int last_k = a.K - (splits - 1) * a.k_per_split;  // K range of the last split
-  if (a.k_per_split / BK < C::STAGES + 2 || last_k / BK < C::STAGES + 2) return launch_gemm<T, C, EPI>(a, splits, st);
+  if (a.k_per_split / BK < C::STAGES + 2 || last_k / BK < C::STAGES + 2) {
+    a.tail_ws = nullptr;
+    return launch_gemm<T, C, EPI>(a, splits, st);
+  }
   const int64_t x_rows = a.top_k > 0 ? a.num_valid / a.top_k : C::BT;
   const int64_t w_rows = EPI == EPI_SILU ? 2 * static_cast<int64_t>(a.N) : a.N;
   const int64_t lim = int64_t(1) << 32, es = sizeof(T);
@@ -307,13 +445,30 @@ int launch_gemm_persistent(const GemmArgs& a, int splits, hipStream_t st) {
   int resident = 0;
   const int rc = persistent_grid<T, C, EPI>(&resident);
   if (rc != FR_OK) return rc;
+  // the fix-up writes whole tiles of 4-column groups: the feature count must be a multiple of the tile's
+  constexpr int COLS = (EPI == EPI_SILU) ? C::BF / 2 : C::BF;
+  const bool tail = a.tail_ws && EPI != EPI_PLAIN && splits == 1 && a.K / BK >= kTailMinTiles && a.N % COLS == 0;
+  if (!tail) a.tail_ws = nullptr;
   const int64_t worst = static_cast<int64_t>(a.num_t_blocks) * a.num_f_tiles;
   int64_t grid = resident / (splits > 1 ? splits : 1) / 8 * 8;  // the splits share the device
   if (grid < 8) grid = 8;
-  if (grid > (worst + 7) / 8 * 8) grid = (worst + 7) / 8 * 8;
+  if (tail) {
+    if (grid > kTailUnits) grid = kTailUnits;  // one slice buffer per workgroup
+  } else if (grid > (worst + 7) / 8 * 8) {
+    grid = (worst + 7) / 8 * 8;
+  }
   hipLaunchKernelGGL((moe_gemm_persistent_kernel<T, C, EPI>), dim3(static_cast<unsigned>(grid), splits), dim3(C::NT),
                      C::LDS_BYTES, st, a);
-  return check_launch("moe_gemm_persistent_kernel");
+  int lrc = check_launch("moe_gemm_persistent_kernel");
+  if (lrc != FR_OK || !tail) return lrc;
+  if constexpr (EPI != EPI_PLAIN) {
+    const int nper = static_cast<int>(grid / 8);
+    if (nper >= 2) {
+      hipLaunchKernelGGL((tail_fixup_kernel<T, C, EPI>), dim3(8 * (nper / 2) * (C::BT / kFixupRows)), dim3(256), 0, st, a, nper);
+      lrc = check_launch("tail_fixup_kernel");
+    }
+  }
+  return lrc;
 }
 
 }  // namespace fr

@@ -48,6 +48,8 @@ def fused_moe(hidden_states: torch.Tensor, gate: torch.Tensor, w1: torch.Tensor,
     align_ws = torch.empty((max(align_bytes, 256),), dtype=torch.uint8, device=dev)
     act = torch.empty((max(p.sorted_len, 1), F), dtype=hidden_states.dtype, device=dev)
     partial = torch.empty((p.split_k * max(n, 1) * K,), dtype=torch.float32, device=dev)
+    tail = torch.empty((p.tail_bytes,), dtype=torch.uint8, device=dev) if p.tail_bytes else None
+    tail_ptr = tail.data_ptr() if tail is not None else None
     out = hidden_states if inplace else torch.empty_like(hidden_states)
     ev[1].record()
 
@@ -60,12 +62,12 @@ def fused_moe(hidden_states: torch.Tensor, gate: torch.Tensor, w1: torch.Tensor,
 
     N.check(lib.fr_moe_gateup_silu(hidden_states.data_ptr(), w1.data_ptr(), sorted_ids.data_ptr(),
                                    expert_ids.data_ptr(), npost.data_ptr(), M, K, F, E, topk, p.block, code,
-                                   act.data_ptr(), st))
+                                   act.data_ptr(), tail_ptr, st))
     ev[4].record()
 
     N.check(lib.fr_moe_down_combine(act.data_ptr(), w2.data_ptr(), topk_weights.data_ptr(), sorted_ids.data_ptr(),
                                     expert_ids.data_ptr(), npost.data_ptr(), M, K, F, E, topk, p.block, p.split_k,
-                                    code, partial.data_ptr(), out.data_ptr(), st))
+                                    code, partial.data_ptr(), out.data_ptr(), tail_ptr, st))
     ev[5].record()
     ev[5].synchronize()
 

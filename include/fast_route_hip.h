@@ -102,6 +102,9 @@ typedef struct fr_moe_plan {
   int32_t split_k;    /* K splits of the down projection                     */
   int64_t sorted_len; /* n + E*(block-1): length of sorted_token_ids         */
   int64_t workspace_bytes; /* bytes fr_fused_moe / fr_fused_experts need     */
+  int64_t tail_bytes; /* bytes of the optional `tail_ws` scratch of the two  */
+                      /* GEMM entry points below (0: the plan has no use for */
+                      /* it); already counted in workspace_bytes             */
 } fr_moe_plan;
 int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk, int dtype, fr_moe_plan* plan);
 
@@ -109,22 +112,28 @@ int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk, int dtype,
  * slot s < num_tokens_post_pad (t = sorted_token_ids[s] / topk, padding slots
  * compute on token 0), written at row s of act[sorted_len, F].
  * Replaces: grouped GEMM 1 + silu_and_mul,
- * fast_route/fast_route/layers/stable_route.py:85-90. */
+ * fast_route/fast_route/layers/stable_route.py:85-90.
+ * `tail_ws`: NULL, or 256-byte aligned device scratch of plan.tail_bytes.  With
+ * it the 256-row tiles that only partly fill the last round of workgroups are
+ * split along K over the idle ones and summed in a fixed order by a second
+ * launch; without it every tile is computed by one workgroup.  Results of the
+ * two modes differ by fp32 summation order only. */
 int fr_moe_gateup_silu(const void* x, const void* w1, const int32_t* sorted_token_ids,
                        const int32_t* expert_ids, const int32_t* num_tokens_post_pad,
                        int64_t M, int64_t H, int64_t F, int E, int topk, int block, int dtype,
-                       void* act, void* stream);
+                       void* act, void* tail_ws, void* stream);
 
 /* out[m, :] = sum_j topk_weights[m, j] * (act[slot(m, j)] @ W2[e]^T), the
  * down projection with the routed weight applied in the GEMM epilogue and the
  * top-k combine.  `partial` is fp32 scratch of split_k * M*topk * H elements.
  * Replaces: grouped GEMM 2 + torch.sum,
- * fast_route/fast_route/layers/stable_route.py:92-102. */
+ * fast_route/fast_route/layers/stable_route.py:92-102.
+ * `tail_ws`: as for fr_moe_gateup_silu (used when split_k == 1). */
 int fr_moe_down_combine(const void* act, const void* w2, const float* topk_weights,
                         const int32_t* sorted_token_ids, const int32_t* expert_ids,
                         const int32_t* num_tokens_post_pad, int64_t M, int64_t H, int64_t F, int E,
                         int topk, int block, int split_k, int dtype, float* partial, void* out,
-                        void* stream);
+                        void* tail_ws, void* stream);
 
 /* Experts only: routing arrays + both GEMMs + combine, from given top-k
  * weights/ids (the fused_moe(hidden, w1, w2, topk_weights, topk_ids) shape of

@@ -120,7 +120,7 @@ def test_token_matrix_of_4gib_is_refused(native):
     dummy = torch.zeros(1 << 16, dtype=torch.int32, device="cuda")
     st = torch.cuda.current_stream().cuda_stream
     rc = N.lib().fr_moe_gateup_silu(dummy.data_ptr(), dummy.data_ptr(), dummy.data_ptr(), dummy.data_ptr(),
-                                    dummy.data_ptr(), M, H, Fd, E, k, block, N.FR_BF16, dummy.data_ptr(), st)
+                                    dummy.data_ptr(), M, H, Fd, E, k, block, N.FR_BF16, dummy.data_ptr(), None, st)
     assert rc == -2, rc
     assert b"4 GiB" in N.lib().fr_last_error_string()
     torch.cuda.synchronize()
@@ -191,6 +191,64 @@ def test_block_256_several_tiles_per_workgroup(native):
     out = fused_moe(xd, w1d, w2d, logits.cuda(), k, True)
     torch.cuda.synchronize()
     _assert_close(out, oracle.fused_moe(x, w1, w2, logits, k, True), dtype, "layer")
+
+
+@pytest.mark.parametrize("case", ["gate_up_after_whole_tile", "down_first_unit", "with_and_without_scratch"])
+def test_last_round_of_tiles_split_along_k(native, case):
+    """256-row tiles that only partly fill the last round of workgroups are cut along K over
+    the idle ones and summed by a second launch.  Routing is constructed so that the tile
+    counts are exact (k = 1, every expert a whole number of 256-token blocks):
+    gate_up_after_whole_tile - 17 blocks x 16 feature tiles = 272 tiles, 34 per XCD: one whole
+      round of 32 and 2 tiles cut into 8 K slices each (K = 4096 is 64 K tiles);
+    down_first_unit - 4 blocks x 2 feature tiles over F = 4096: 1 tile per XCD in 8 slices,
+      the slice being the workgroup's first and only unit;
+    with_and_without_scratch - the two GEMM entry points with and without the scratch agree
+      to fp32 summation order (same bf16 result up to one rounding)."""
+    from fast_route_amd import _native as N, fused_experts
+    from fast_route_amd.layers.fused_moe import plan
+    _say("tail split " + case)
+    dtype = torch.bfloat16
+    if case == "down_first_unit":
+        H, Fd, E, blocks = 512, 4096, 2, (3, 1)
+    else:
+        H, Fd, E, blocks = 4096, 2048, 3, (9, 0, 8)
+    M = 256 * sum(blocks)
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(M, H, generator=g).to(dtype)
+    w1 = (torch.randn(E, 2 * Fd, H, generator=g) * 0.02).to(dtype)
+    w2 = (torch.randn(E, H, Fd, generator=g) * 0.02).to(dtype)
+    ids = torch.cat([torch.full((256 * b,), e, dtype=torch.int32) for e, b in enumerate(blocks)])
+    ids = ids[torch.randperm(M, generator=g)].view(M, 1)
+    w = (torch.rand(M, 1, generator=g) + 0.5).float()
+    p = plan(M, H, Fd, E, 1, dtype)
+    assert p.block == 256 and p.tail_bytes > 0 and p.split_k == 1
+    xd, w1d, w2d, wd, idd = x.cuda(), w1.cuda(), w2.cuda(), w.cuda(), ids.cuda()
+    if case != "with_and_without_scratch":
+        out = fused_experts(xd, w1d, w2d, wd, idd)
+        torch.cuda.synchronize()
+        _assert_close(out, oracle.moe_experts(x, w1, w2, w, ids), dtype, case)
+        return
+    from fast_route_amd.ops.fused_moe import moe_align_block_size
+    lib, st = N.lib(), torch.cuda.current_stream().cuda_stream
+    s, e, npost = moe_align_block_size(idd, 256, E)
+    tail = torch.empty(p.tail_bytes, dtype=torch.uint8, device="cuda")
+    res = []
+    for tptr in (None, tail.data_ptr()):
+        act = torch.zeros(s.numel(), Fd, dtype=dtype, device="cuda")
+        partial = torch.empty(M * H, dtype=torch.float32, device="cuda")
+        out = torch.empty(M, H, dtype=dtype, device="cuda")
+        N.check(lib.fr_moe_gateup_silu(xd.data_ptr(), w1d.data_ptr(), s.data_ptr(), e.data_ptr(), npost.data_ptr(), M, H,
+                                       Fd, E, 1, 256, N.FR_BF16, act.data_ptr(), tptr, st))
+        N.check(lib.fr_moe_down_combine(act.data_ptr(), w2d.data_ptr(), wd.data_ptr(), s.data_ptr(), e.data_ptr(),
+                                        npost.data_ptr(), M, H, Fd, E, 1, 256, 1, N.FR_BF16, partial.data_ptr(),
+                                        out.data_ptr(), tptr, st))
+        torch.cuda.synchronize()
+        res.append((act.float().cpu(), out.float().cpu()))
+    (act0, out0), (act1, out1) = res
+    assert not torch.equal(act0, act1), "the scratch changed nothing: the split path did not run"
+    # one bf16 rounding apart at most (2^-8 relative), on values whose fp32 sums differ in the last bits
+    assert ((act0 - act1).abs() <= 2.0 ** -7 * act0.abs().clamp(min=1e-3)).all()
+    assert ((out0 - out1).abs() <= 2.0 ** -6 * out0.abs().max()).all()
 
 
 def test_stable_and_vllm_route_layers(native):
