@@ -94,8 +94,8 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // tiles are cut along K over the idle workgroups); both GEMMs share the scratch for that.
   const int64_t tail_up = tail_scratch_bytes(block, dtype, H, F, true), tail_down = tail_scratch_bytes(block, dtype, F, H, false);
   int split = 1;
-  if (tail_down > 0) {
-    split = 1;
+  if (tail_down > 0 && tiles >= 192) {
+    split = 1;  // whole rounds plus a split last round; below, too few tiles for one round: split them all
   } else if (block >= 128) {
     // one workgroup per CU: pick the split whose grid fills whole rounds of 256 CUs best,
     // charging 7 % per extra fp32 partial slice (its write + re-read in the combine)

@@ -38,6 +38,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
 template <typename T> struct Tiles {  // bf16 / fp16
   typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
+  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0> T128P;  // persistent form (down projection)
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
   typedef Cfg<32, 128, 128, 1, 4, 16, 2, 3> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
@@ -77,7 +78,12 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       // its neighbour's.  The fp8 fragments leave no registers for the second address set.
       if constexpr (sizeof(T) == 2) return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
       else return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
-    case 128: fill(128, TL::T128::BF, TL::T128::BKB); return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
+    case 128:
+      fill(128, TL::T128::BF, TL::T128::BKB);
+      // The down projection has few feature tiles and a long K: it gains from the persistent form's
+      // split of the last round; the gate/up GEMM at these sizes streams weights and does not.
+      if constexpr (sizeof(T) == 2 && EPI == EPI_DOWN) return launch_gemm_persistent<T, typename TL::T128P, EPI>(a, splits, st);
+      else return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
     case 64: fill(64, TL::T64::BF, TL::T64::BKB); return launch_gemm<T, typename TL::T64, EPI>(a, splits, st);
     case 32:
       if (EPI == EPI_SILU && a.K % (TL::T32L::BKB / static_cast<int>(sizeof(T))) == 0) {
@@ -129,11 +135,12 @@ int usable_splits(int split_k, int64_t K, int bk) {
 }
 
 int64_t tail_scratch_bytes(int block, int dtype, int64_t K, int64_t N, bool gateup) {
-  typedef Tiles<bf16_t>::T256 C;  // the one tile that runs persistently (2-byte operands only)
-  if (block != 256 || (dtype != FR_BF16 && dtype != FR_F16)) return 0;
+  typedef Tiles<bf16_t>::T256 C;  // the tiles that run persistently (2-byte operands only): T256, and T128P for the down GEMM
+  static_assert(Tiles<bf16_t>::T128P::BF == C::BF && Tiles<bf16_t>::T128P::BKB == C::BKB, "same K tile and feature tile");
+  if (!(block == 256 || (block == 128 && !gateup)) || (dtype != FR_BF16 && dtype != FR_F16)) return 0;
   const int64_t bk = C::BKB / 2, cols = gateup ? C::BF / 2 : C::BF;
   if (K / bk < kTailMinTiles || N % cols != 0) return 0;
-  return static_cast<int64_t>(kTailUnits) * C::BT * C::BF * 4;
+  return static_cast<int64_t>(kTailUnits) * C::BT * C::BF * 4;  // sized for the larger tile
 }
 
 int gateup_impl(const void* x, const float* x_scale, const void* w1, const float* w1_scale,
