@@ -4,10 +4,14 @@
 namespace fr {
 
 // ---- top-k combine: out[m] = sum over splits and slots of partial ------------
-template <typename T>
-__global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ partial,
+// P = float (one fp32 slice per K split) or the operand type (single slice: each pair's row
+// rounded once before the sum over its token's slots, as the reference's second GEMM writes it,
+// fast_route/fast_route/ops/fused_moe.py:117-123, before torch.sum).
+template <typename T, typename P>
+__global__ __launch_bounds__(256) void combine_kernel(const P* __restrict__ partial,
                                                       int64_t split_stride, int splits, int topk,
                                                       int64_t M, int H, T* __restrict__ out) {
+  typedef P p4 __attribute__((ext_vector_type(4)));
   const int64_t idx = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
   if (idx >= M * H) return;
   const int64_t m = idx / H;
@@ -15,8 +19,9 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
   f32x4 s = {0.f, 0.f, 0.f, 0.f};
   for (int j = 0; j < topk; ++j)
     for (int sp = 0; sp < splits; ++sp) {
-      const f32x4 v = *reinterpret_cast<const f32x4*>(partial + sp * split_stride + (m * topk + j) * H + h);
-      s += v;
+      const p4 v = *reinterpret_cast<const p4*>(partial + sp * split_stride + (m * topk + j) * H + h);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[r] += static_cast<float>(v[r]);
     }
   typename Elem<T>::out4 o;
 #pragma unroll
@@ -82,8 +87,10 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       fill(128, TL::T128::BF, TL::T128::BKB);
       // The down projection has few feature tiles and a long K: it gains from the persistent form's
       // split of the last round; the gate/up GEMM at these sizes streams weights and does not.
-      if constexpr (sizeof(T) == 2 && EPI == EPI_DOWN) return launch_gemm_persistent<T, typename TL::T128P, EPI>(a, splits, st);
-      else return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
+      if constexpr (sizeof(T) == 2 && EPI != EPI_SILU) {
+        if (a.long_k) return launch_gemm_persistent<T, typename TL::T128P, EPI>(a, splits, st);
+      }
+      return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
     case 64: fill(64, TL::T64::BF, TL::T64::BKB); return launch_gemm<T, typename TL::T64, EPI>(a, splits, st);
     case 32:
       if (EPI == EPI_SILU && a.K % (TL::T32L::BKB / static_cast<int>(sizeof(T))) == 0) {
@@ -114,16 +121,32 @@ int dispatch_dtype(const GemmArgs& a, int dtype, int block, int splits, int64_t 
   return fail(FR_E_DTYPE, "dtype %d not in {f16, bf16, fp8_e4m3}", dtype);
 }
 
-int launch_combine(const float* partial, int64_t split_stride, int splits, int topk, int64_t M, int H,
+template <typename T, typename P>
+void launch_combine_as(const void* partial, int64_t split_stride, int splits, int topk, int64_t M, int H, void* out,
+                       hipStream_t st) {
+  const unsigned grid = static_cast<unsigned>(ceil_div(M * H / 4, 256));
+  hipLaunchKernelGGL((combine_kernel<T, P>), dim3(grid), dim3(256), 0, st, static_cast<const P*>(partial), split_stride,
+                     splits, topk, M, H, static_cast<T*>(out));
+}
+
+// partial_dtype: FR_F32, or the 2-byte type a single slice was written in
+int launch_combine(const void* partial, int partial_dtype, int64_t split_stride, int splits, int topk, int64_t M, int H,
                    int out_dtype, void* out, hipStream_t st) {
   if (M == 0) return FR_OK;
-  const unsigned grid = static_cast<unsigned>(ceil_div(M * H / 4, 256));
-  if (out_dtype == FR_BF16)
-    hipLaunchKernelGGL(combine_kernel<bf16_t>, dim3(grid), dim3(256), 0, st, partial, split_stride, splits, topk, M, H, static_cast<bf16_t*>(out));
-  else if (out_dtype == FR_F16)
-    hipLaunchKernelGGL(combine_kernel<f16_t>, dim3(grid), dim3(256), 0, st, partial, split_stride, splits, topk, M, H, static_cast<f16_t*>(out));
-  else
-    return fail(FR_E_DTYPE, "output dtype %d not in {f16, bf16}", out_dtype);
+  if (out_dtype != FR_BF16 && out_dtype != FR_F16) return fail(FR_E_DTYPE, "output dtype %d not in {f16, bf16}", out_dtype);
+  const bool ob = out_dtype == FR_BF16;
+  if (partial_dtype == FR_F32) {
+    if (ob) launch_combine_as<bf16_t, float>(partial, split_stride, splits, topk, M, H, out, st);
+    else launch_combine_as<f16_t, float>(partial, split_stride, splits, topk, M, H, out, st);
+  } else if (partial_dtype == FR_BF16) {
+    if (ob) launch_combine_as<bf16_t, bf16_t>(partial, split_stride, splits, topk, M, H, out, st);
+    else launch_combine_as<f16_t, bf16_t>(partial, split_stride, splits, topk, M, H, out, st);
+  } else if (partial_dtype == FR_F16) {
+    if (ob) launch_combine_as<bf16_t, f16_t>(partial, split_stride, splits, topk, M, H, out, st);
+    else launch_combine_as<f16_t, f16_t>(partial, split_stride, splits, topk, M, H, out, st);
+  } else {
+    return fail(FR_E_DTYPE, "partial dtype %d", partial_dtype);
+  }
   return check_launch("combine_kernel");
 }
 
@@ -153,7 +176,7 @@ int gateup_impl(const void* x, const float* x_scale, const void* w1, const float
   FR_REQUIRE(H > 0 && H % k_multiple(dtype, block) == 0, FR_E_SHAPE, "%s: H=%lld must be a multiple of %d for block %d", who, (long long)H, k_multiple(dtype, block), block);
   FR_REQUIRE(F > 0 && F % 8 == 0, FR_E_SHAPE, "%s: F=%lld must be a positive multiple of 8", who, (long long)F);
   FR_REQUIRE(topk >= 1 && E >= 1 && M * topk < (int64_t(1) << 30), FR_E_SHAPE, "%s: M*topk too large", who);
-  FR_REQUIRE(aligned16(x) && aligned16(w1) && aligned16(act), FR_E_ALIGN, "%s: operands must be 16-byte aligned", who);
+  FR_REQUIRE(aligned16(x) && aligned16(w1) && aligned16(act) && aligned16(tail_ws), FR_E_ALIGN, "%s: operands must be 16-byte aligned", who);
   const int64_t n = M * topk, sorted_len = n + int64_t(E) * (block - 1);
   GemmArgs a = {};
   a.X = x; a.ldx = H; a.W = w1; a.w_expert_stride = 2 * F * H; a.ldw = H; a.out = act; a.ldo = F;
@@ -175,7 +198,7 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
   FR_REQUIRE(H > 0 && H % 4 == 0, FR_E_SHAPE, "%s: H=%lld must be a positive multiple of 4", who, (long long)H);
   FR_REQUIRE(split_k >= 1 && split_k <= 64, FR_E_SHAPE, "%s: split_k=%d outside [1, 64]", who, split_k);
   FR_REQUIRE(topk >= 1 && E >= 1 && M * topk < (int64_t(1) << 30), FR_E_SHAPE, "%s: M*topk too large", who);
-  FR_REQUIRE(aligned16(act) && aligned16(w2) && aligned16(partial) && aligned16(out), FR_E_ALIGN, "%s: operands must be 16-byte aligned", who);
+  FR_REQUIRE(aligned16(act) && aligned16(w2) && aligned16(partial) && aligned16(out) && aligned16(tail_ws), FR_E_ALIGN, "%s: operands must be 16-byte aligned", who);
   const int64_t n = M * topk, sorted_len = n + int64_t(E) * (block - 1);
   const int splits = usable_splits(split_k, F, k_multiple(dtype, block));
   GemmArgs a = {};
@@ -186,9 +209,16 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
   a.topk_w = topk_weights; a.num_valid = (int)n; a.top_k = 0; a.N = (int)H; a.K = (int)F;
   a.mul_weight = 1;
   a.tail_ws = tail_ws;
+  a.long_k = 1;
+  if (splits == 1) {
+    // one slice: each pair's row in the operands' 2-byte type (bf16 for fp8 operands), half the partial traffic
+    int rc = dispatch_dtype<EPI_PLAIN>(a, dtype, block, 1, sorted_len / block * block, st);
+    if (rc != FR_OK) return rc;
+    return launch_combine(partial, dtype == FR_F16 ? FR_F16 : FR_BF16, n * H, 1, topk, M, (int)H, out_dtype, out, st);
+  }
   int rc = dispatch_dtype<EPI_DOWN>(a, dtype, block, splits, sorted_len / block * block, st);
   if (rc != FR_OK) return rc;
-  return launch_combine(partial, n * H, splits, topk, M, (int)H, out_dtype, out, st);
+  return launch_combine(partial, FR_F32, n * H, splits, topk, M, (int)H, out_dtype, out, st);
 }
 
 }  // namespace fr

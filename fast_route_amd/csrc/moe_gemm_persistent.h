@@ -348,8 +348,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 }
 
 // Sums the K slices of the tiles of each XCD's last round in slice order and applies the
-// epilogue the GEMM would have applied: routed weight and scatter to the pair's row of the
-// fp32 partial buffer (EPI_DOWN), or silu(gate)*up to the slot's row of act (EPI_SILU).
+// epilogue the GEMM would have applied: routed weight and scatter to the pair's row (EPI_DOWN
+// in fp32, EPI_PLAIN in the operand type), or silu(gate)*up to the slot's row of act (EPI_SILU).
 // Grid: 8 XCDs x nper/2 tiles (a split tail has at most that many) x BT/32 row groups; blocks
 // without a split tile leave at once.  nper = workgroups per XCD of the GEMM launch.
 constexpr int kFixupRows = 32;
@@ -358,7 +358,6 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(const GemmArgs a, int n
   typedef Elem<T> E;
   typedef typename E::out_t out_t;
   typedef typename E::out4 out4;
-  static_assert(EPI == EPI_SILU || EPI == EPI_DOWN, "fix-up of the fused epilogues only");
   constexpr int BT = C::BT, BF = C::BF, BK = C::BKB / static_cast<int>(sizeof(T));
   constexpr int COLS = (EPI == EPI_SILU) ? BF / 2 : BF;  // output columns of a tile
   constexpr int CG = COLS / 4, RPP = 256 / CG;           // 4-column groups per row, rows per pass
@@ -379,15 +378,22 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(const GemmArgs a, int n
     const int row = rb * kFixupRows + p * RPP + threadIdx.x / CG;
     const int slot = pid_t * BT + row;
     const float* src = first + row * BF + cg * 4;
-    if constexpr (EPI == EPI_DOWN) {
+    if constexpr (EPI != EPI_SILU) {
       const int sid = a.sorted[slot];
       if (sid >= a.num_valid) continue;
       f32x4 sum = *reinterpret_cast<const f32x4*>(src);
       for (int s = 1; s < xs.slices; ++s) sum += *reinterpret_cast<const f32x4*>(src + s * slice_stride);
       const float rw = a.mul_weight ? a.topk_w[sid] : 1.f;
-      float* orow = static_cast<float*>(a.out) + static_cast<int64_t>(sid) * a.ldo + pid_f * BF + cg * 4;
-      const f32x4 o = {sum[0] * rw, sum[1] * rw, sum[2] * rw, sum[3] * rw};
-      *reinterpret_cast<f32x4*>(orow) = o;
+      const int64_t at = static_cast<int64_t>(sid) * a.ldo + pid_f * BF + cg * 4;
+      if constexpr (EPI == EPI_DOWN) {
+        const f32x4 o = {sum[0] * rw, sum[1] * rw, sum[2] * rw, sum[3] * rw};
+        *reinterpret_cast<f32x4*>(static_cast<float*>(a.out) + at) = o;
+      } else {
+        out4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = static_cast<out_t>(sum[r] * rw);
+        *reinterpret_cast<out4*>(static_cast<out_t*>(a.out) + at) = o;
+      }
     } else {
       f32x4 g = *reinterpret_cast<const f32x4*>(src), u = *reinterpret_cast<const f32x4*>(src + BF / 2);
       for (int s = 1; s < xs.slices; ++s) {
@@ -403,25 +409,27 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(const GemmArgs a, int n
   }
 }
 
-// Workgroups resident at once on the device (a multiple of 8, one share per XCD).
+// Workgroups resident at once on the current device (a multiple of 8, one share per XCD).
 template <typename T, typename C, int EPI>
 int persistent_grid(int* grid_out) {
-  static int cached = 0;
-  if (!cached) {
-    hipError_t e = hipSuccess;
+  constexpr int kMaxDevices = 64;
+  static int cached[kMaxDevices] = {};  // per device; a race between threads writes the same value twice
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(FR_E_LAUNCH, "persistent GEMM: device %d (%s)", dev, hipGetErrorString(e));
+  if (!cached[dev]) {
     if (C::LDS_BYTES > 65536)
       e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_persistent_kernel<T, C, EPI>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    int dev = 0, cus = 0, per_cu = 0;
-    if (e == hipSuccess) e = hipGetDevice(&dev);
+    int cus = 0, per_cu = 0;
     if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e == hipSuccess)
       e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, moe_gemm_persistent_kernel<T, C, EPI>, C::NT, C::LDS_BYTES);
     if (e != hipSuccess) return fail(FR_E_LAUNCH, "persistent GEMM set-up (%d B LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
     if (per_cu < 1 || cus < 8) return fail(FR_E_LAUNCH, "persistent GEMM: occupancy %d on %d CUs", per_cu, cus);
-    cached = cus * per_cu / 8 * 8;
+    cached[dev] = cus * per_cu / 8 * 8;
   }
-  *grid_out = cached;
+  *grid_out = cached[dev];
   return FR_OK;
 }
 
@@ -447,7 +455,7 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
   if (rc != FR_OK) return rc;
   // the fix-up writes whole tiles of 4-column groups: the feature count must be a multiple of the tile's
   constexpr int COLS = (EPI == EPI_SILU) ? C::BF / 2 : C::BF;
-  const bool tail = a.tail_ws && EPI != EPI_PLAIN && splits == 1 && a.K / BK >= kTailMinTiles && a.N % COLS == 0;
+  const bool tail = a.tail_ws && splits == 1 && a.K / BK >= kTailMinTiles && a.N % COLS == 0;
   if (!tail) a.tail_ws = nullptr;
   const int64_t worst = static_cast<int64_t>(a.num_t_blocks) * a.num_f_tiles;
   int64_t grid = resident / (splits > 1 ? splits : 1) / 8 * 8;  // the splits share the device
@@ -461,12 +469,10 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
                      C::LDS_BYTES, st, a);
   int lrc = check_launch("moe_gemm_persistent_kernel");
   if (lrc != FR_OK || !tail) return lrc;
-  if constexpr (EPI != EPI_PLAIN) {
-    const int nper = static_cast<int>(grid / 8);
-    if (nper >= 2) {
-      hipLaunchKernelGGL((tail_fixup_kernel<T, C, EPI>), dim3(8 * (nper / 2) * (C::BT / kFixupRows)), dim3(256), 0, st, a, nper);
-      lrc = check_launch("tail_fixup_kernel");
-    }
+  const int nper = static_cast<int>(grid / 8);
+  if (nper >= 2) {
+    hipLaunchKernelGGL((tail_fixup_kernel<T, C, EPI>), dim3(8 * (nper / 2) * (C::BT / kFixupRows)), dim3(256), 0, st, a, nper);
+    lrc = check_launch("tail_fixup_kernel");
   }
   return lrc;
 }

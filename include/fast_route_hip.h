@@ -125,7 +125,8 @@ int fr_moe_gateup_silu(const void* x, const void* w1, const int32_t* sorted_toke
 
 /* out[m, :] = sum_j topk_weights[m, j] * (act[slot(m, j)] @ W2[e]^T), the
  * down projection with the routed weight applied in the GEMM epilogue and the
- * top-k combine.  `partial` is fp32 scratch of split_k * M*topk * H elements.
+ * top-k combine.  `partial` is scratch of split_k * M*topk * H floats (with
+ * split_k == 1 only its first half is used: the pairs' rows are kept in `dtype`).
  * Replaces: grouped GEMM 2 + torch.sum,
  * fast_route/fast_route/layers/stable_route.py:92-102.
  * `tail_ws`: as for fr_moe_gateup_silu (used when split_k == 1). */
