@@ -118,7 +118,8 @@ class Layer:
             N.check(lib.fr_moe_down_combine_fp8(self.actq.data_ptr(), self.acts.data_ptr(), w2q.data_ptr(), w2s.data_ptr(),
                                                 self.tw.data_ptr(), self.sorted.data_ptr(), self.eids.data_ptr(),
                                                 self.npost.data_ptr(), self.M, self.H, self.F, self.E, self.topk, p.block,
-                                                p.split_k, N.FR_BF16, self.partial.data_ptr(), self.out.data_ptr(), self.stream))
+                                                p.split_k, N.FR_BF16, self.partial.data_ptr(), self.out.data_ptr(),
+                                                self.tail.data_ptr() if self.tail is not None else None, self.stream))
             rec(4)
             return
         N.check(lib.fr_moe_gateup_silu(self.x.data_ptr(), self.w1.data_ptr(), self.sorted.data_ptr(), self.eids.data_ptr(),

@@ -40,7 +40,7 @@ SIGNATURES = {
                                        c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p]),
     "fr_moe_down_combine_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p,
-                                        c_void_p, c_void_p]),
+                                        c_void_p, c_void_p, c_void_p]),
     "fr_fused_moe_fp8": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64,
                                  c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_void_p]),
     "fr_fused_moe": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int,

@@ -193,5 +193,5 @@ extern "C" int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, con
   rc = quant_rows(c.act, FR_BF16, p.sorted_len, c.npost, F, F, c.actq, c.act_scale, st);
   if (rc != FR_OK) return rc;
   return fr_moe_down_combine_fp8(c.actq, c.act_scale, w2q, w2_scale, c.topk_w, c.sorted, c.expert_ids, c.npost, M, H, F, E,
-                                 topk, p.block, p.split_k, x_dtype, c.partial, out, stream);
+                                 topk, p.block, p.split_k, x_dtype, c.partial, out, c.tail, stream);
 }

@@ -53,6 +53,7 @@ template <typename T> struct Tiles {  // bf16 / fp16
 template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per two K-steps
   typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
+  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0> T128P;
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
   typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
@@ -81,13 +82,18 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       fill(256, TL::T256::BF, TL::T256::BKB);
       // One workgroup per CU: the persistent form hides each tile's ring fill and drain behind
       // its neighbour's.  The fp8 fragments leave no registers for the second address set.
-      if constexpr (sizeof(T) == 2) return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
-      else return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
+      if constexpr (sizeof(T) == 2) {
+        return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
+      } else if constexpr (EPI != EPI_SILU) {
+        // fp8: no hand-off between tiles, but the down projection still gains the split of its last round
+        if (a.long_k) return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
+      }
+      return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
     case 128:
       fill(128, TL::T128::BF, TL::T128::BKB);
       // The down projection has few feature tiles and a long K: it gains from the persistent form's
       // split of the last round; the gate/up GEMM at these sizes streams weights and does not.
-      if constexpr (sizeof(T) == 2 && EPI != EPI_SILU) {
+      if constexpr (EPI != EPI_SILU) {
         if (a.long_k) return launch_gemm_persistent<T, typename TL::T128P, EPI>(a, splits, st);
       }
       return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
@@ -158,10 +164,15 @@ int usable_splits(int split_k, int64_t K, int bk) {
 }
 
 int64_t tail_scratch_bytes(int block, int dtype, int64_t K, int64_t N, bool gateup) {
-  typedef Tiles<bf16_t>::T256 C;  // the tiles that run persistently (2-byte operands only): T256, and T128P for the down GEMM
+  // The tiles that run persistently: T256 (both GEMMs for 2-byte operands, the down projection for fp8)
+  // and T128P (down projection).  Same K bytes per tile and same feature tile in all of them.
+  typedef Tiles<bf16_t>::T256 C;
   static_assert(Tiles<bf16_t>::T128P::BF == C::BF && Tiles<bf16_t>::T128P::BKB == C::BKB, "same K tile and feature tile");
-  if (!(block == 256 || (block == 128 && !gateup)) || (dtype != FR_BF16 && dtype != FR_F16)) return 0;
-  const int64_t bk = C::BKB / 2, cols = gateup ? C::BF / 2 : C::BF;
+  static_assert(Tiles<fp8_t>::T256::BF == C::BF && Tiles<fp8_t>::T256::BKB == C::BKB, "same K tile and feature tile");
+  const bool two_byte = dtype == FR_BF16 || dtype == FR_F16;
+  if (!two_byte && dtype != FR_FP8_E4M3) return 0;
+  if (!((block == 256 && (two_byte || !gateup)) || (block == 128 && !gateup))) return 0;
+  const int64_t bk = C::BKB / elem_bytes(dtype), cols = gateup ? C::BF / 2 : C::BF;
   if (K / bk < kTailMinTiles || N % cols != 0) return 0;
   return static_cast<int64_t>(kTailUnits) * C::BT * C::BF * 4;  // sized for the larger tile
 }
@@ -282,9 +293,9 @@ extern "C" int fr_moe_down_combine_fp8(const void* actq, const float* act_scale,
                                        const float* topk_weights, const int32_t* sorted_token_ids,
                                        const int32_t* expert_ids, const int32_t* num_tokens_post_pad, int64_t M,
                                        int64_t H, int64_t F, int E, int topk, int block, int split_k, int out_dtype,
-                                       float* partial, void* out, void* stream) {
+                                       float* partial, void* out, void* tail_ws, void* stream) {
   FR_REQUIRE(act_scale && w2_scale, FR_E_NULL, "fr_moe_down_combine_fp8: null scale pointer");
   return down_impl(actq, act_scale, w2q, w2_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, M,
-                   H, F, E, topk, block, split_k, FR_FP8_E4M3, out_dtype, partial, out, nullptr,
+                   H, F, E, topk, block, split_k, FR_FP8_E4M3, out_dtype, partial, out, static_cast<float*>(tail_ws),
                    static_cast<hipStream_t>(stream), "fr_moe_down_combine_fp8");
 }

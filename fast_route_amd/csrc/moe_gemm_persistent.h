@@ -98,6 +98,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
   constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, IW = C::IW, NLI = (XI + WI) * IW;
   constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
+  constexpr bool HANDOFF = !E::SCALED;  // the 8-register fp8 fragments leave no room for a second address set
   static_assert(S >= 2 && C::SPREAD <= 1, "persistent form: ring of at least two slots, refill in one group");
   static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
   static_assert((S - 1) * NLI <= 63, "vmcnt budget");
@@ -315,27 +316,48 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     if (tu < 0) gemm_epilogue<T, C, EPI>(a, acc, pid_t, pid_f, expert, split, wt, wf, frow, kgrp);         \
     else tail_store<C, EPI>(a.tail_ws + static_cast<int64_t>(xcd * nper + tu) * (BT * BF), acc, wt, wf, frow, kgrp); \
   }
-  // Whole pipeline for an issuing (ISS_ = true) or a non-issuing wavefront.
-#define FR_PERSIST(ISS_)                                                                                   \
+  // Fill of the ring with the first S K tiles of set A and the first fragments.
+#define FR_FILL(ISS_)                                                                                      \
   {                                                                                                        \
     _Pragma("unroll") for (int t = 0; t < S; ++t)                                                          \
       if (ISS_) { _Pragma("unroll") for (int q = 0; q < NLI; ++q) FR_ISSUE_ONE(A, t, t, q); }               \
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((S - 1) * NLI) : "memory");                                   \
     __builtin_amdgcn_s_barrier();                                                                          \
     FR_READ_FRAGS(0, 0, 0);                                                                                \
+  }
+  // Whole pipeline for an issuing (ISS_ = true) or a non-issuing wavefront.  HANDOFF: the ring
+  // passes from unit to unit as described above; without it (fp8: no registers for the second
+  // address set) every unit fills and drains the ring by itself.
+#define FR_PERSIST(ISS_)                                                                                   \
+  {                                                                                                        \
+    FR_FILL(ISS_)                                                                                          \
     int sl = 0;                                                                                            \
     int unit = 0;                                                                                          \
-    for (; unit + 1 < n_units; ++unit) { /* a next unit exists: hand the ring over to it */                \
-      FR_TILE(ISS_, true)                                                                                  \
-      pid_t = n_pid_t; pid_f = n_pid_f; expert = n_expert; xrsA = xrsB; wrsA = wrsB;                       \
-      kb = n_kb; kn = n_kn; tu = n_tu;                                                                     \
-      _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) xsrcA[ih] = xsrcB[ih];                        \
-      _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) wsrcA[ih] = wsrcB[ih];                        \
+    if constexpr (HANDOFF) {                                                                               \
+      for (; unit + 1 < n_units; ++unit) { /* a next unit exists: hand the ring over to it */              \
+        FR_TILE(ISS_, true)                                                                                \
+        pid_t = n_pid_t; pid_f = n_pid_f; expert = n_expert; xrsA = xrsB; wrsA = wrsB;                     \
+        kb = n_kb; kn = n_kn; tu = n_tu;                                                                   \
+        _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) xsrcA[ih] = xsrcB[ih];                      \
+        _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) wsrcA[ih] = wsrcB[ih];                      \
+      }                                                                                                    \
+      FR_TILE(ISS_, false)                                                                                 \
+    } else {                                                                                               \
+      for (;;) {                                                                                           \
+        FR_TILE(ISS_, false)                                                                               \
+        if (++unit == n_units) break;                                                                      \
+        FR_UNIT(unit, pid_t, pid_f, kb, kn, tu)                                                            \
+        expert = a.expert_ids[pid_t];                                                                      \
+        FR_MAKE_SET(pid_t, pid_f, expert, kb, a.sorted[pid_t * BT + rr], xsrcA, wsrcA, xrsA, wrsA)         \
+        __syncthreads(); /* every wavefront is done with the ring before it is filled again */            \
+        FR_FILL(ISS_)                                                                                      \
+        sl = 0;                                                                                            \
+      }                                                                                                    \
     }                                                                                                      \
-    FR_TILE(ISS_, false)                                                                                   \
   }
   if (IW == 1 || issuer) FR_PERSIST(true) else FR_PERSIST(false)
 #undef FR_PERSIST
+#undef FR_FILL
 #undef FR_TILE
 #undef FR_KTILE
 #undef FR_KSTEP
@@ -370,6 +392,8 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(const GemmArgs a, int n
   if (xs.slices < 2 || t >= xs.rest) return;
   int pid_t, pid_f;
   tile_coords(a, nt, xs.base + xs.rounds * nper + t, pid_t, pid_f);
+  const float* wsc = nullptr;
+  if constexpr (E::SCALED) wsc = a.w_scale + static_cast<int64_t>(a.expert_ids[pid_t]) * a.w_rows;
   const float* first = a.tail_ws + static_cast<int64_t>(xcd * nper + t) * (BT * BF);
   const int64_t slice_stride = static_cast<int64_t>(xs.rest) * (BT * BF);
   const int cg = threadIdx.x % CG;
@@ -383,7 +407,12 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(const GemmArgs a, int n
       if (sid >= a.num_valid) continue;
       f32x4 sum = *reinterpret_cast<const f32x4*>(src);
       for (int s = 1; s < xs.slices; ++s) sum += *reinterpret_cast<const f32x4*>(src + s * slice_stride);
-      const float rw = a.mul_weight ? a.topk_w[sid] : 1.f;
+      float rw = a.mul_weight ? a.topk_w[sid] : 1.f;
+      if constexpr (E::SCALED) {  // per-row scales of both fp8 operands
+        rw *= a.top_k > 0 ? a.x_scale[sid / a.top_k] : a.x_scale[slot];
+        const f32x4 ws = *reinterpret_cast<const f32x4*>(wsc + pid_f * BF + cg * 4);
+        sum *= ws;
+      }
       const int64_t at = static_cast<int64_t>(sid) * a.ldo + pid_f * BF + cg * 4;
       if constexpr (EPI == EPI_DOWN) {
         const f32x4 o = {sum[0] * rw, sum[1] * rw, sum[2] * rw, sum[3] * rw};
@@ -399,6 +428,14 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(const GemmArgs a, int n
       for (int s = 1; s < xs.slices; ++s) {
         g += *reinterpret_cast<const f32x4*>(src + s * slice_stride);
         u += *reinterpret_cast<const f32x4*>(src + s * slice_stride + BF / 2);
+      }
+      if constexpr (E::SCALED) {
+        const int sid = a.sorted[slot];
+        const float xsc = a.top_k > 0 ? (sid < a.num_valid ? a.x_scale[sid / a.top_k] : 1.f) : a.x_scale[slot];
+        const f32x4 gs = *reinterpret_cast<const f32x4*>(wsc + pid_f * (BF / 2) + cg * 4);
+        const f32x4 us = *reinterpret_cast<const f32x4*>(wsc + a.N + pid_f * (BF / 2) + cg * 4);
+        g *= gs * xsc;
+        u *= us * xsc;
       }
       out4 o;
 #pragma unroll

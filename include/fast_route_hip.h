@@ -169,7 +169,7 @@ int fr_quant_e4m3_rows(const void* x, int dtype, int64_t rows, int64_t K, int64_
 /* fp8 forms of fr_moe_gateup_silu / fr_moe_down_combine: operands are e4m3
  * codes with one fp32 scale per row (x_scale[M], w1_scale[E, 2F], act_scale
  * [sorted_len], w2_scale[E, H]); act is written / read in bf16 resp. e4m3;
- * H and F must be multiples of 256. */
+ * H and F must be multiples of 256.  `tail_ws` as for fr_moe_down_combine. */
 int fr_moe_gateup_silu_fp8(const void* xq, const float* x_scale, const void* w1q, const float* w1_scale,
                            const int32_t* sorted_token_ids, const int32_t* expert_ids,
                            const int32_t* num_tokens_post_pad, int64_t M, int64_t H, int64_t F, int E,
@@ -178,7 +178,7 @@ int fr_moe_down_combine_fp8(const void* actq, const float* act_scale, const void
                             const float* topk_weights, const int32_t* sorted_token_ids,
                             const int32_t* expert_ids, const int32_t* num_tokens_post_pad, int64_t M,
                             int64_t H, int64_t F, int E, int topk, int block, int split_k, int out_dtype,
-                            float* partial, void* out, void* stream);
+                            float* partial, void* out, void* tail_ws, void* stream);
 
 /* Whole fp8 layer from bf16 activations and router logits: gating, routing,
  * per-token quantisation of x, fp8 gate/up GEMM + SiLU*mul (bf16 act), per-row

@@ -67,7 +67,9 @@ def test_fp8_layer_vs_oracle(native, M):
 
 
 def test_fp8_mixtral_shape_sampled(native):
-    """Full fp8 workload shape (H4096 F14336 E8 top2), M in {16, 256}: sampled tokens vs the oracle."""
+    """Full fp8 workload shape (H4096 F14336 E8 top2), M in {16, 256, 4096}: sampled tokens vs the
+    oracle.  At M=4096 the down projection runs the persistent form with its last round of tiles
+    split along K."""
     from fast_route_amd import fused_moe_fp8, prepare_weights_fp8
     H, Fd, E, k = 4096, 14336, 8, 2
     g = torch.Generator(device="cuda").manual_seed(5)
@@ -75,7 +77,7 @@ def test_fp8_mixtral_shape_sampled(native):
     w2 = (torch.randn(E, H, Fd, generator=g, device="cuda") * 0.02).bfloat16()
     w1q, w1s, w2q, w2s = prepare_weights_fp8(w1, w2)
     w1c, w2c = w1.cpu(), w2.cpu()
-    for M in (16, 256):
+    for M in (16, 256, 4096):
         _say(f"fp8 mixtral M={M}")
         x = torch.randn(M, H, generator=g, device="cuda").bfloat16()
         logits = torch.randn(M, E, generator=g, device="cuda")
@@ -87,3 +89,31 @@ def test_fp8_mixtral_shape_sampled(native):
         assert (o - ref).norm() / ref.norm() <= 1e-2
         out2 = fused_moe_fp8(x, w1q, w1s, w2q, w2s, logits, k, True)
         assert torch.equal(out, out2)
+
+
+def test_fp8_down_projection_tail_split(native):
+    """Routing built so that the down projection has 4 token blocks x 2 feature tiles of 256 rows
+    over K = 4096: one tile per XCD, cut into 8 K slices whose sum the fix-up kernel scales
+    (activation-row scale x weight-row scale x routed weight) and rounds."""
+    from fast_route_amd import fused_moe_fp8, prepare_weights_fp8
+    from fast_route_amd.layers.fused_moe import plan
+    from fast_route_amd import _native as N
+    _say("fp8 tail split")
+    H, Fd, E, k, M = 512, 4096, 2, 1, 1024
+    p = plan(M, H, Fd, E, k, torch.bfloat16, code=N.FR_FP8_E4M3)
+    assert p.block == 256 and p.tail_bytes > 0 and p.split_k == 1
+    g = torch.Generator().manual_seed(91)
+    x = torch.randn(M, H, generator=g).bfloat16()
+    w1 = (torch.randn(E, 2 * Fd, H, generator=g) * 0.02).bfloat16()
+    w2 = (torch.randn(E, H, Fd, generator=g) * 0.02).bfloat16()
+    ids = torch.cat([torch.zeros(768, dtype=torch.long), torch.ones(256, dtype=torch.long)])[torch.randperm(M, generator=g)]
+    logits = torch.full((M, E), -4.0)
+    logits[torch.arange(M), ids] = 4.0
+    w1q, w1s, w2q, w2s = prepare_weights_fp8(w1.cuda(), w2.cuda())
+    out = fused_moe_fp8(x.cuda(), w1q, w1s, w2q, w2s, logits.cuda(), k, True)
+    torch.cuda.synchronize()
+    ref, _ = oracle.fused_moe_fp8(x, w1, w2, logits, k, True)
+    o = out.float().cpu()
+    assert torch.isfinite(o).all()
+    assert (o - ref).norm() / ref.norm() <= 1e-2
+    assert (o - ref).abs().max() <= 2.0 ** -5 * ref.abs().max()
