@@ -492,7 +492,9 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
   if (rc != FR_OK) return rc;
   // the fix-up writes whole tiles of 4-column groups: the feature count must be a multiple of the tile's
   constexpr int COLS = (EPI == EPI_SILU) ? C::BF / 2 : C::BF;
-  const bool tail = a.tail_ws && splits == 1 && a.K / BK >= kTailMinTiles && a.N % COLS == 0;
+  // tiles the fix-up's thread map covers: 4-column groups of a row over 256 threads, 32-row groups
+  constexpr bool kFixable = C::BT % kFixupRows == 0 && 256 % (COLS / 4) == 0 && kFixupRows % (256 / (COLS / 4)) == 0;
+  const bool tail = kFixable && a.tail_ws && splits == 1 && a.K / BK >= kTailMinTiles && a.N % COLS == 0;
   if (!tail) a.tail_ws = nullptr;
   const int64_t worst = static_cast<int64_t>(a.num_t_blocks) * a.num_f_tiles;
   int64_t grid = resident / (splits > 1 ? splits : 1) / 8 * 8;  // the splits share the device
@@ -506,10 +508,12 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
                      C::LDS_BYTES, st, a);
   int lrc = check_launch("moe_gemm_persistent_kernel");
   if (lrc != FR_OK || !tail) return lrc;
-  const int nper = static_cast<int>(grid / 8);
-  if (nper >= 2) {
-    hipLaunchKernelGGL((tail_fixup_kernel<T, C, EPI>), dim3(8 * (nper / 2) * (C::BT / kFixupRows)), dim3(256), 0, st, a, nper);
-    lrc = check_launch("tail_fixup_kernel");
+  if constexpr (kFixable) {
+    const int nper = static_cast<int>(grid / 8);
+    if (nper >= 2) {
+      hipLaunchKernelGGL((tail_fixup_kernel<T, C, EPI>), dim3(8 * (nper / 2) * (C::BT / kFixupRows)), dim3(256), 0, st, a, nper);
+      lrc = check_launch("tail_fixup_kernel");
+    }
   }
   return lrc;
 }
