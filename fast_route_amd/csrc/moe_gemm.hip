@@ -83,11 +83,10 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       // One workgroup per CU: the persistent form hides each tile's ring fill and drain behind
       // its neighbour's.  The fp8 fragments leave no registers for the second address set.
       if constexpr (sizeof(T) == 2) {
-        // Walk order of the persistent gate/up GEMM: with few token blocks, all of them per feature tile (a
-        // weight tile then serves every block of its expert at once and is fetched once; the token rows,
-        // 2 MB per block, stay in L2/MALL); with many, groups of 8.  Measured at M = 2048 / 4096 / 16384:
-        // -4 % / -2 % / -0.5 % against groups of 4.
-        if (EPI == EPI_SILU) a.group_t = a.num_t_blocks <= 40 ? a.num_t_blocks : 8;
+        // Walk order of the persistent gate/up GEMM: groups of 8 token blocks once there are many (-3.4 % at
+        // M = 8192, -0.8 % at 16384 against groups of 4).  Walking ALL token blocks per feature tile is another
+        // 1 % faster at M <= 4096 but fetches 65 % more through L2 (token rows re-read per feature tile): not taken.
+        if (EPI == EPI_SILU && a.num_t_blocks > 40) a.group_t = 8;
         return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
       } else if constexpr (EPI != EPI_SILU) {
         // fp8: no hand-off between tiles, but the down projection still gains the split of its last round
