@@ -83,10 +83,6 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       // One workgroup per CU: the persistent form hides each tile's ring fill and drain behind
       // its neighbour's.  The fp8 fragments leave no registers for the second address set.
       if constexpr (sizeof(T) == 2) {
-        // Walk order of the persistent gate/up GEMM: groups of 8 token blocks once there are many (-3.4 % at
-        // M = 8192, -0.8 % at 16384 against groups of 4).  Walking ALL token blocks per feature tile is another
-        // 1 % faster at M <= 4096 but fetches 65 % more through L2 (token rows re-read per feature tile): not taken.
-        if (EPI == EPI_SILU && a.num_t_blocks > 40) a.group_t = 8;
         return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
       } else if constexpr (EPI != EPI_SILU) {
         // fp8: no hand-off between tiles, but the down projection still gains the split of its last round
@@ -198,6 +194,7 @@ int gateup_impl(const void* x, const float* x_scale, const void* w1, const float
   a.sorted = sorted; a.expert_ids = expert_ids; a.npost = npost;
   a.x_scale = x_scale; a.w_scale = w1_scale; a.w_rows = static_cast<int>(2 * F);
   a.num_valid = (int)n; a.top_k = topk; a.N = (int)F; a.K = (int)H;
+  a.num_experts = E;
   a.tail_ws = tail_ws;
   return dispatch_dtype<EPI_SILU>(a, dtype, block, 1, sorted_len / block * block, st);
 }
@@ -223,6 +220,7 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
   a.x_scale = act_scale; a.w_scale = w2_scale; a.w_rows = static_cast<int>(H);
   a.topk_w = topk_weights; a.num_valid = (int)n; a.top_k = 0; a.N = (int)H; a.K = (int)F;
   a.mul_weight = 1;
+  a.num_experts = E;
   a.tail_ws = tail_ws;
   a.long_k = 1;
   if (splits == 1) {
@@ -260,6 +258,7 @@ extern "C" int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, vo
   a.sorted = sorted_token_ids; a.expert_ids = expert_ids; a.npost = num_tokens_post_pad;
   a.topk_w = topk_weights; a.num_valid = (int)num_valid; a.top_k = top_k; a.N = (int)N; a.K = (int)K;
   a.mul_weight = mul_routed_weight;
+  a.num_experts = E;
   // only whole blocks inside sorted_token_ids are addressable
   return dispatch_dtype<EPI_PLAIN>(a, dtype, block, 1, sorted_len / block * block, static_cast<hipStream_t>(stream));
 }

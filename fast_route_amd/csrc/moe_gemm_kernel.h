@@ -47,6 +47,7 @@ struct GemmArgs {
   int num_f_tiles;
   int group_t;
   int mul_weight;
+  int num_experts;      // E (persistent form: walk order by expert)
   int long_k;           // down projection (few feature tiles, long K): hint for the 128-row tile's form
   float* tail_ws;       // persistent form only: slice buffers for splitting the last round of tiles along K, or nullptr
 };

@@ -50,13 +50,51 @@ __device__ __forceinline__ XcdSchedule xcd_schedule(int total, int nper, int xcd
   }
   return s;
 }
-// Walk order of the tiles: groups of group_t token blocks x all feature tiles.
-__device__ __forceinline__ void tile_coords(const GemmArgs& a, int nt, int lin, int& pid_t, int& pid_f) {
-  const int in_group = a.group_t * a.num_f_tiles;
-  const int first = (lin / in_group) * a.group_t;
-  const int gsz = min(nt - first, a.group_t);
-  pid_t = first + (lin % in_group) % gsz;
-  pid_f = (lin % in_group) / gsz;
+// Walk order of the tiles.  The token blocks of one expert are consecutive (the routing sort is by
+// expert), and only they use that expert's weight tiles.  Tiles are therefore ordered expert by
+// expert; an expert's run of blocks is cut into equal chunks of at most group_t blocks and a chunk
+// is walked block-fastest over all feature tiles.  Consecutive tiles - the ones an XCD's workgroups
+// hold at any moment - then share one expert's weight tiles and a few token blocks, and a weight
+// tile is fetched by one chunk only (groups of a fixed number of blocks straddle experts and fetch
+// two experts' tiles each: measured 4.6 GB through L2 per launch against 2.1 GB of operands).
+constexpr int kMaxExperts = 1024;  // limit of the routing entry points
+constexpr int kChunkBlocks = 8;    // token blocks per chunk, at most (measured 4 / 8 / 16: 1675 / 1648 / 1640 us at M=4096,
+                                   // 8 and 12 best at M=16384)
+// off[e] = first token block of expert e among the nt real blocks (expert_ids ascends), off[E] = nt
+__device__ __forceinline__ void expert_block_offsets(const GemmArgs& a, int nt, int* off, int tid, int nthreads) {
+  for (int e = tid; e <= a.num_experts; e += nthreads) {
+    int lo = 0, hi = nt;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (a.expert_ids[mid] < e) lo = mid + 1;
+      else hi = mid;
+    }
+    off[e] = lo;
+  }
+}
+__device__ __forceinline__ void tile_coords(const GemmArgs& a, const int* off, int lin, int& pid_t, int& pid_f,
+                                            int& expert) {
+  const int F = a.num_f_tiles;
+  expert = a.expert_ids[lin / F];  // lin / F is one of the expert's blocks: its tiles are [off[e] * F, off[e + 1] * F)
+  const int first = off[expert], len = off[expert + 1] - first;
+  const int chunks = (len + a.group_t - 1) / a.group_t, base = len / chunks, rem = len - base * chunks;
+  int q = lin - first * F;
+  const int big = rem * (base + 1) * F;  // the first rem chunks hold one block more
+  int gsz, start;
+  if (q < big) {
+    gsz = base + 1;
+    const int c = q / (gsz * F);
+    q -= c * gsz * F;
+    start = first + c * gsz;
+  } else {
+    q -= big;
+    gsz = base;
+    const int c = q / (gsz * F);
+    q -= c * gsz * F;
+    start = first + rem * (base + 1) + c * gsz;
+  }
+  pid_t = start + q % gsz;
+  pid_f = q / gsz;
 }
 // Tile column of accumulator tile j of feature wavefront wf (= row of the weight tile in LDS).
 template <typename C, int EPI>
@@ -112,7 +150,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   // ---- schedule ---------------------------------------------------------------
   // The real tile count is dealt to the 8 XCDs (workgroup id mod 8) in contiguous ranges; the
   // workgroups of one XCD take the tiles of its range round robin, so at any moment they work on
-  // consecutive tiles (group_t token blocks x consecutive feature tiles: shared in that XCD's L2).
+  // consecutive tiles (see tile_coords: a few token blocks of one expert x consecutive feature tiles,
+  // shared in that XCD's L2).
   // Work unit j of a workgroup: tile j of its round-robin walk over all K tiles, or, after the
   // whole rounds, one K slice of a tile of the last round.
   const int npost = a.npost[0];
@@ -125,6 +164,9 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   const XcdSchedule xs = xcd_schedule(total, nper, xcd, k_all, a.tail_ws != nullptr);
   const int n_units = xs.rounds + (loc < xs.rest * xs.slices ? 1 : 0);
   if (n_units == 0) return;
+  __shared__ int expert_off[kMaxExperts + 1];
+  expert_block_offsets(a, nt, expert_off, threadIdx.x, C::NT);
+  __syncthreads();
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wt = wave / C::WF, wf = wave % C::WF;
@@ -133,7 +175,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   const T* X = static_cast<const T*>(a.X);
 
   // unit j_ -> tile coordinates, first K tile kb_ and K tile count kn_, slice buffer tu_ (-1: a whole tile)
-#define FR_UNIT(j_, pt_, pf_, kb_, kn_, tu_)                                                   \
+#define FR_UNIT(j_, pt_, pf_, ex_, kb_, kn_, tu_)                                              \
   {                                                                                            \
     int lin_;                                                                                  \
     if ((j_) < xs.rounds) {                                                                    \
@@ -146,7 +188,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
       kn_ = (s_ + 1) * k_all / xs.slices - kb_;                                                \
       tu_ = xs.slices > 1 ? s_ * xs.rest + t_ : -1;                                            \
     }                                                                                          \
-    tile_coords(a, nt, lin_, pt_, pf_);                                                        \
+    tile_coords(a, expert_off, lin_, pt_, pf_, ex_);                                           \
   }
   // rows of the load slots this wavefront issues: load index ih -> tile row
 #define FR_SLOT_ROW(ih_, rr_, c_)                                                  \
@@ -209,8 +251,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
                                         static_cast<int64_t>(sizeof(T)));                                    \
     }                                                                                                        \
   }
-  FR_UNIT(0, pid_t, pid_f, kb, kn, tu)
-  expert = a.expert_ids[pid_t];
+  FR_UNIT(0, pid_t, pid_f, expert, kb, kn, tu)
   FR_MAKE_SET(pid_t, pid_f, expert, kb, a.sorted[pid_t * BT + rr], xsrcA, wsrcA, xrsA, wrsA)
 
   // load q_ of an issuing wavefront (weight-tile loads first) of K tile tile_ into ring slot slot_
@@ -288,8 +329,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #define FR_TILE(ISS_, NEXT)                                                                                \
   {                                                                                                        \
     if (NEXT) {                                                                                            \
-      FR_UNIT(unit + 1, n_pid_t, n_pid_f, n_kb, n_kn, n_tu)                                                \
-      n_expert = a.expert_ids[n_pid_t];                                                                    \
+      FR_UNIT(unit + 1, n_pid_t, n_pid_f, n_expert, n_kb, n_kn, n_tu)                                      \
       if (a.top_k > 0) {                                                                                   \
         _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) {                                           \
           FR_SLOT_ROW(ih, rr, c)                                                                           \
@@ -346,8 +386,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
       for (;;) {                                                                                           \
         FR_TILE(ISS_, false)                                                                               \
         if (++unit == n_units) break;                                                                      \
-        FR_UNIT(unit, pid_t, pid_f, kb, kn, tu)                                                            \
-        expert = a.expert_ids[pid_t];                                                                      \
+        FR_UNIT(unit, pid_t, pid_f, expert, kb, kn, tu)                                                    \
         FR_MAKE_SET(pid_t, pid_f, expert, kb, a.sorted[pid_t * BT + rr], xsrcA, wsrcA, xrsA, wrsA)         \
         __syncthreads(); /* every wavefront is done with the ring before it is filled again */            \
         FR_FILL(ISS_)                                                                                      \
@@ -390,10 +429,13 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(const GemmArgs a, int n
   const int nt = min(a.npost[0] / BT, a.num_t_blocks);
   const XcdSchedule xs = xcd_schedule(nt * a.num_f_tiles, nper, xcd, a.K / BK, true);
   if (xs.slices < 2 || t >= xs.rest) return;
-  int pid_t, pid_f;
-  tile_coords(a, nt, xs.base + xs.rounds * nper + t, pid_t, pid_f);
+  __shared__ int expert_off[kMaxExperts + 1];
+  expert_block_offsets(a, nt, expert_off, threadIdx.x, 256);
+  __syncthreads();
+  int pid_t, pid_f, expert;
+  tile_coords(a, expert_off, xs.base + xs.rounds * nper + t, pid_t, pid_f, expert);
   const float* wsc = nullptr;
-  if constexpr (E::SCALED) wsc = a.w_scale + static_cast<int64_t>(a.expert_ids[pid_t]) * a.w_rows;
+  if constexpr (E::SCALED) wsc = a.w_scale + static_cast<int64_t>(expert) * a.w_rows;
   const float* first = a.tail_ws + static_cast<int64_t>(xcd * nper + t) * (BT * BF);
   const int64_t slice_stride = static_cast<int64_t>(xs.rest) * (BT * BF);
   const int cg = threadIdx.x % CG;
@@ -477,7 +519,7 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
   GemmArgs a = a_in;
   constexpr int BK = C::BKB / static_cast<int>(sizeof(T));
   const int last_k = a.K - (splits - 1) * a.k_per_split;  // K range of the last split
-  if (a.k_per_split / BK < C::STAGES + 2 || last_k / BK < C::STAGES + 2) {
+  if (a.k_per_split / BK < C::STAGES + 2 || last_k / BK < C::STAGES + 2 || a.num_experts < 1 || a.num_experts > kMaxExperts) {
     a.tail_ws = nullptr;
     return launch_gemm<T, C, EPI>(a, splits, st);
   }
@@ -487,6 +529,7 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
   if (x_rows * a.ldx * es >= lim || w_rows * a.ldw * es >= lim)
     return fail(FR_E_SHAPE, "token rows (%lld x %lld) or one expert's weights (%lld x %lld) span 4 GiB or more",
                 (long long)x_rows, (long long)a.ldx, (long long)w_rows, (long long)a.ldw);
+  a.group_t = kChunkBlocks;
   int resident = 0;
   const int rc = persistent_grid<T, C, EPI>(&resident);
   if (rc != FR_OK) return rc;
