@@ -80,10 +80,14 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // Routing block = token rows per GEMM tile.  Decode sizes want one block per expert
   // (weights are streamed once); from ~32 pairs per expert on, the 128-row MFMA tile
   // wins even with its padding, and 256 rows once runs are long enough to amortise it.
+  // The 256-row tile's advantage grows with the K of the gate/up GEMM (its start-up per
+  // tile is amortised over more K tiles); measured crossovers: 352..384 pairs per expert
+  // at H = 4096 (F = 14336, E = 8), 576..768 at H = 2048 (F = 1408, E = 64).
+  const double t256 = H >= 4096 ? 368.0 : (H <= 2048 ? 640.0 : 640.0 - (H - 2048) * (272.0 / 2048.0));
   int block;
   if (avg <= 8) block = 16;
-  else if (avg <= 32) block = 32;
-  else if (avg < 320) block = 128;
+  else if (avg < 32) block = 32;
+  else if (avg < t256) block = 128;
   else block = 256;
   // Down projection: N = H gives few feature tiles, so K is split.
   const int bf = block == 16 ? 64 : (block == 32 ? 128 : 256);
@@ -94,17 +98,22 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // tiles are cut along K over the idle workgroups); both GEMMs share the scratch for that.
   const int64_t tail_up = tail_scratch_bytes(block, dtype, H, F, true), tail_down = tail_scratch_bytes(block, dtype, F, H, false);
   int split = 1;
-  if (tail_down > 0 && tiles >= 192) {
-    split = 1;  // whole rounds plus a split last round; below, too few tiles for one round: split them all
+  if (tail_down > 0 && (tiles >= 192 || tiles <= 64)) {
+    // whole rounds plus a split last round, or so few tiles that every one is cut into 4..8 slices;
+    // in between (most of one round: no idle workgroups to cut for) all tiles are split alike
   } else if (block >= 128) {
-    // one workgroup per CU: pick the split whose grid fills whole rounds of 256 CUs best,
-    // charging 7 % per extra fp32 partial slice (its write + re-read in the combine)
-    double best = -1.0;
+    // one workgroup per CU: the split that minimises GEMM time (how well tiles x split fill whole rounds
+    // of 256 CUs, at ~0.9 PFLOP/s) plus the partial traffic it causes (one 2-byte slice, or `split` fp32
+    // slices, written and read back at ~4 TB/s: with many pairs per weight byte that traffic decides)
+    double best = 1e30;
+    const double rows = static_cast<double>(blocks) * block, pairs = static_cast<double>(n);
     for (int sp = 1; sp <= 4; ++sp) {
       if (F / sp < 8 * bk_elems) break;
       const double work = static_cast<double>(tiles) * sp;
-      const double eff = work / (256.0 * static_cast<double>(ceil_div(tiles * sp, 256))) - 0.07 * (sp - 1);
-      if (eff > best) { best = eff; split = sp; }
+      const double fill = work / (256.0 * static_cast<double>(ceil_div(tiles * sp, 256)));
+      const double t_gemm = 2.0 * rows * H * F / 0.9e15 / fill;
+      const double t_part = pairs * H * (sp == 1 ? 2.0 : 4.0 * sp) * 2.0 / 4e12;
+      if (t_gemm + t_part < best) { best = t_gemm + t_part; split = sp; }
     }
   } else {
     // several workgroups per CU: aim at ~512 workgroups

@@ -92,21 +92,21 @@ def test_fp8_mixtral_shape_sampled(native):
 
 
 def test_fp8_down_projection_tail_split(native):
-    """Routing built so that the down projection has 4 token blocks x 2 feature tiles of 256 rows
-    over K = 4096: one tile per XCD, cut into 8 K slices whose sum the fix-up kernel scales
+    """Routing built so that the down projection has 8 token blocks x 2 feature tiles of 256 rows
+    over K = 4096: two tiles per XCD, each cut into 8 K slices whose sum the fix-up kernel scales
     (activation-row scale x weight-row scale x routed weight) and rounds."""
     from fast_route_amd import fused_moe_fp8, prepare_weights_fp8
     from fast_route_amd.layers.fused_moe import plan
     from fast_route_amd import _native as N
     _say("fp8 tail split")
-    H, Fd, E, k, M = 512, 4096, 2, 1, 1024
+    H, Fd, E, k, M = 512, 4096, 2, 1, 2048
     p = plan(M, H, Fd, E, k, torch.bfloat16, code=N.FR_FP8_E4M3)
     assert p.block == 256 and p.tail_bytes > 0 and p.split_k == 1
     g = torch.Generator().manual_seed(91)
     x = torch.randn(M, H, generator=g).bfloat16()
     w1 = (torch.randn(E, 2 * Fd, H, generator=g) * 0.02).bfloat16()
     w2 = (torch.randn(E, H, Fd, generator=g) * 0.02).bfloat16()
-    ids = torch.cat([torch.zeros(768, dtype=torch.long), torch.ones(256, dtype=torch.long)])[torch.randperm(M, generator=g)]
+    ids = torch.cat([torch.zeros(1280, dtype=torch.long), torch.ones(768, dtype=torch.long)])[torch.randperm(M, generator=g)]
     logits = torch.full((M, E), -4.0)
     logits[torch.arange(M), ids] = 4.0
     w1q, w1s, w2q, w2s = prepare_weights_fp8(w1.cuda(), w2.cuda())

@@ -200,8 +200,8 @@ def test_last_round_of_tiles_split_along_k(native, case):
     counts are exact (k = 1, every expert a whole number of 256-token blocks):
     gate_up_after_whole_tile - 17 blocks x 16 feature tiles = 272 tiles, 34 per XCD: one whole
       round of 32 and 2 tiles cut into 8 K slices each (K = 4096 is 64 K tiles);
-    down_first_unit - 4 blocks x 2 feature tiles over F = 4096: 1 tile per XCD in 8 slices,
-      the slice being the workgroup's first and only unit;
+    down_first_unit - 8 blocks x 2 feature tiles over F = 4096: 2 tiles per XCD in 8 slices
+      each, the slice being the workgroup's first and only unit;
     with_and_without_scratch - the two GEMM entry points with and without the scratch agree
       to fp32 summation order (same bf16 result up to one rounding)."""
     from fast_route_amd import _native as N, fused_experts
@@ -209,7 +209,7 @@ def test_last_round_of_tiles_split_along_k(native, case):
     _say("tail split " + case)
     dtype = torch.bfloat16
     if case == "down_first_unit":
-        H, Fd, E, blocks = 512, 4096, 2, (3, 1)
+        H, Fd, E, blocks = 512, 4096, 2, (5, 3)
     else:
         H, Fd, E, blocks = 4096, 2048, 3, (9, 0, 8)
     M = 256 * sum(blocks)
