@@ -57,13 +57,14 @@ __global__ __launch_bounds__(kGateThreads) void gating_topk_blocked_kernel(
 }
 
 // ---- gate-matrix form: logits tile by MFMA, then the same gating -------------
-// One workgroup owns kRgTokens tokens (16 per wavefront).  The gate matrix is
-// [H, E] with experts contiguous, so each K tile of it is transposed through
-// LDS into expert-major rows that the MFMA "A" operand can read as 16-byte
-// vectors; token rows come straight from HBM as the "B" operand.
-constexpr int kRgTokens = 64;
-constexpr int kRgBK = 64;
-constexpr int kRgPitch = kRgBK + 8;  // elements; keeps 16-byte alignment, spreads banks
+// The token rows [M, H] are the only real traffic (the gate matrix, [H, E] with experts
+// contiguous, stays in L2), so the kernel is shaped to stream them: a workgroup of 4
+// wavefronts owns 64 tokens (16 per wavefront), or, while there are too few tokens to fill
+// the CUs that way, 16 tokens whose K range the 4 wavefronts split and reduce through LDS.
+// The gate is taken in chunks of kRgKC rows, each transposed once through registers into
+// expert-major LDS rows (two K rows packed per 32-bit store) that the MFMA "A" operand reads
+// as 16-byte vectors; token rows come straight from HBM as the "B" operand, fetched for the
+// whole chunk before the barrier that publishes it.
 constexpr int kRgMaxE = 64;
 
 template <typename T> struct Mfma16;
@@ -76,63 +77,112 @@ template <> struct Mfma16<f16_t> {
   static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
 };
 
-template <typename T, int G>
+// KC = K rows of the gate per LDS chunk; TT = 16-token tiles per wavefront in the unsplit form (many
+// experts: more tokens per transposed gate chunk).
+template <typename T, int G, bool SPLITK, int KC, int TT>
 __global__ __launch_bounds__(kGateThreads) void route_gate_kernel(
     const T* __restrict__ hidden, const T* __restrict__ gate, int64_t M, int H, int E, int topk,
     int renorm, float* __restrict__ w_out, int32_t* __restrict__ ids_out) {
   typedef typename Mfma16<T>::vec8 vec8;
-  constexpr int ET = (G + 15) / 16;  // expert tiles of 16
-  __shared__ __attribute__((aligned(16))) T gt[ET * 16 * kRgPitch];
-  __shared__ float logit[kRgTokens * (kRgMaxE + 1)];
+  static_assert(kGateThreads == 256, "4 wavefronts");
+  static_assert(!SPLITK || TT == 1, "the split form has one token tile");
+  constexpr int ET = (G + 15) / 16;              // expert tiles of 16
+  constexpr int TPC = SPLITK ? 16 : 64 * TT;     // tokens per workgroup
+  constexpr int KW = SPLITK ? KC / 4 : KC;       // K elements of a chunk one wavefront multiplies
+  constexpr int KSTEPS = KW / 32;
+  constexpr int PITCH = KC + 8;                  // elements; keeps 16-byte alignment, spreads banks
+  constexpr int LP = ET * 16 + 1;                // pitch of a logit row (floats)
+  __shared__ __attribute__((aligned(16))) T gt[ET * 16 * PITCH];
+  __shared__ float logit[TPC * LP];
+  __shared__ float part[SPLITK ? 4 * 16 * LP : 1];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * kRgTokens;
-  const int64_t my_tok = tok0 + wave * 16 + (lane & 15);
-  const T* xrow = hidden + (my_tok < M ? my_tok : 0) * H + (lane >> 4) * 8;
+  const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * TPC;
+  const int kw0 = SPLITK ? wave * KW : 0;        // the wavefront's K range inside a chunk
+  int trow[TT];                                  // the lane's tokens inside the workgroup
+  const T* xrow[TT];
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    trow[t] = (SPLITK ? 0 : (wave * TT + t) * 16) + (lane & 15);
+    const int64_t tok = tok0 + trow[t];
+    xrow[t] = hidden + (tok < M ? tok : 0) * H + kw0 + (lane >> 4) * 8;
+  }
 
-  for (int i = tid; i < ET * 16 * kRgPitch; i += kGateThreads) gt[i] = static_cast<T>(0.f);
-  f32x4 acc[ET];
+  for (int i = tid; i < ET * 16 * PITCH; i += kGateThreads) gt[i] = static_cast<T>(0.f);  // experts >= E stay 0
+  f32x4 acc[TT][ET];
 #pragma unroll
-  for (int j = 0; j < ET; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < TT; ++t)
+#pragma unroll
+    for (int j = 0; j < ET; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bool vec_gate = E % 8 == 0 && (reinterpret_cast<uintptr_t>(gate) & 15u) == 0;
 
-  for (int k0 = 0; k0 < H; k0 += kRgBK) {
-    __syncthreads();
-    const int kmax = min(kRgBK, H - k0);
-    for (int i = tid; i < kmax * E; i += kGateThreads) {
-      const int k = i / E, e = i % E;
-      gt[e * kRgPitch + k] = gate[static_cast<int64_t>(k0 + k) * E + e];
-    }
-    if (kmax < kRgBK)
-      for (int i = tid; i < (kRgBK - kmax) * E; i += kGateThreads) gt[(i % E) * kRgPitch + kmax + i / E] = static_cast<T>(0.f);
-    __syncthreads();
+  for (int kc = 0; kc < H; kc += KC) {
+    vec8 xf[TT][KSTEPS];
 #pragma unroll
-    for (int ks = 0; ks < kRgBK / 32; ++ks) {
-      const int kk = k0 + ks * 32 + (lane >> 4) * 8;
-      vec8 xf;
-      if (kk + 8 <= H) xf = *reinterpret_cast<const vec8*>(xrow + k0 + ks * 32);
-      else
+    for (int t = 0; t < TT; ++t)
 #pragma unroll
-        for (int r = 0; r < 8; ++r) xf[r] = static_cast<T>(0.f);
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int kk = kc + kw0 + ks * 32 + (lane >> 4) * 8;
+        if (kk + 8 <= H) xf[t][ks] = *reinterpret_cast<const vec8*>(xrow[t] + kc + ks * 32);
+        else
 #pragma unroll
-      for (int j = 0; j < ET; ++j) {
-        const vec8 gf = *reinterpret_cast<const vec8*>(&gt[(j * 16 + (lane & 15)) * kRgPitch + ks * 32 + (lane >> 4) * 8]);
-        acc[j] = Mfma16<T>::mma(gf, xf, acc[j]);
+          for (int r = 0; r < 8; ++r) xf[t][ks][r] = static_cast<T>(0.f);
+      }
+    __syncthreads();  // the previous chunk has been read
+    if (vec_gate) {
+      // item = (pair of K rows, 8 experts): two 16-byte loads, eight 32-bit stores of (k, k+1) pairs
+      const int evs = E / 8;
+      for (int item = tid; item < (KC / 2) * evs; item += kGateThreads) {
+        const int kp = item % (KC / 2), ev = item / (KC / 2);
+        const int k = kc + 2 * kp;
+        vec8 r0, r1;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) { r0[r] = static_cast<T>(0.f); r1[r] = static_cast<T>(0.f); }
+        if (k < H) r0 = *reinterpret_cast<const vec8*>(gate + static_cast<int64_t>(k) * E + ev * 8);
+        if (k + 1 < H) r1 = *reinterpret_cast<const vec8*>(gate + static_cast<int64_t>(k + 1) * E + ev * 8);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          typedef T pair_t __attribute__((ext_vector_type(2)));
+          const pair_t pr = {r0[r], r1[r]};
+          *reinterpret_cast<pair_t*>(&gt[(ev * 8 + r) * PITCH + 2 * kp]) = pr;
+        }
+      }
+    } else {
+      for (int i = tid; i < KC * E; i += kGateThreads) {
+        const int k = i / E, e = i % E;
+        gt[e * PITCH + k] = kc + k < H ? gate[static_cast<int64_t>(kc + k) * E + e] : static_cast<T>(0.f);
       }
     }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+      for (int j = 0; j < ET; ++j) {
+        const vec8 gf = *reinterpret_cast<const vec8*>(&gt[(j * 16 + (lane & 15)) * PITCH + kw0 + ks * 32 + (lane >> 4) * 8]);
+#pragma unroll
+        for (int t = 0; t < TT; ++t) acc[t][j] = Mfma16<T>::mma(gf, xf[t][ks], acc[t][j]);
+      }
   }
   // accumulator rows are experts (lane/16*4 + r inside tile j), columns tokens
+  float* dst = SPLITK ? part + wave * 16 * LP : logit;
 #pragma unroll
-  for (int j = 0; j < ET; ++j)
+  for (int t = 0; t < TT; ++t)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int e = j * 16 + (lane >> 4) * 4 + r;
-      if (e < E) logit[(wave * 16 + (lane & 15)) * (kRgMaxE + 1) + e] = acc[j][r];
-    }
+    for (int j = 0; j < ET; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) dst[trow[t] * LP + j * 16 + (lane >> 4) * 4 + r] = acc[t][j][r];
   __syncthreads();
+  if constexpr (SPLITK) {
+    for (int i = tid; i < 16 * ET * 16; i += kGateThreads) {
+      const int t = i / (ET * 16), e = i % (ET * 16);
+      logit[t * LP + e] = (part[t * LP + e] + part[(16 + t) * LP + e]) + (part[(32 + t) * LP + e] + part[(48 + t) * LP + e]);
+    }
+    __syncthreads();
+  }
   constexpr int PER_PASS = kGateThreads / G;
-  for (int t = tid / G; t < kRgTokens; t += PER_PASS) {
+  for (int t = tid / G; t < TPC; t += PER_PASS) {
     const int64_t token = tok0 + t;
     const bool live = token < M;
-    const float* row = logit + t * (kRgMaxE + 1);
+    const float* row = logit + t * LP;
     gate_token<G, 1>([&](int e) { return row[e]; }, live, E, topk, renorm, w_out + token * topk,
                      ids_out + token * topk);
   }
@@ -213,9 +263,18 @@ namespace {
 template <typename T, int G>
 void launch_route_gate(const void* hidden, const void* gate, int64_t M, int H, int E, int topk, int renorm,
                        float* w, int32_t* ids, hipStream_t st) {
-  const unsigned grid = static_cast<unsigned>(ceil_div(M, kRgTokens));
-  hipLaunchKernelGGL((route_gate_kernel<T, G>), dim3(grid), dim3(kGateThreads), 0, st,
-                     static_cast<const T*>(hidden), static_cast<const T*>(gate), M, H, E, topk, renorm, w, ids);
+  constexpr int ET = (G + 15) / 16;
+  // 64 (128 with many experts) tokens per workgroup once that gives every CU a workgroup or two; below,
+  // 16 tokens with K split over the wavefronts (more workgroups, a quarter of the row per wavefront)
+  if (M >= 16384) {
+    constexpr int TT = ET >= 2 ? 2 : 1;
+    hipLaunchKernelGGL((route_gate_kernel<T, G, false, 256, TT>), dim3(static_cast<unsigned>(ceil_div(M, 64 * TT))), dim3(kGateThreads),
+                       0, st, static_cast<const T*>(hidden), static_cast<const T*>(gate), M, H, E, topk, renorm, w, ids);
+  } else {
+    constexpr int KC = 256;  // longer chunks for few experts leave fewer workgroups per CU: slower at M = 8192, no gain at M = 1
+    hipLaunchKernelGGL((route_gate_kernel<T, G, true, KC, 1>), dim3(static_cast<unsigned>(ceil_div(M, 16))), dim3(kGateThreads), 0, st,
+                       static_cast<const T*>(hidden), static_cast<const T*>(gate), M, H, E, topk, renorm, w, ids);
+  }
 }
 template <typename T>
 int dispatch_route_gate(const void* hidden, const void* gate, int64_t M, int H, int E, int topk, int renorm,
