@@ -52,6 +52,22 @@ __global__ __launch_bounds__(kQuantThreads) void quant_rows_kernel(const T* __re
   amax = wave_max(amax);
   const float s = amax > 0.f ? amax / 448.f : 1.f;
   if (lane == 0) scale[row] = s;
+  // x / s for every element of the row.  With y = RN(1/s), q = RN(x*y), r = x - s*q (exact in an
+  // FMA), RN(q + r*y) is the correctly rounded quotient (Markstein) as long as nothing leaves the
+  // normal range: rows with 2^-40 <= max|x| <= 2^40 take this 3-instruction form - there an
+  // element below 2^-70, whose r could be subnormal, has |x/s| < 2^-21 and encodes as zero either
+  // way - and any other row the IEEE division (10 instructions per element, which made this
+  // kernel ALU bound).  Checked against exact rational arithmetic on 7e5 bf16/fp16 pairs.
+  const bool fast = amax >= 0x1p-40f && amax <= 0x1p40f;
+  const float y = 1.f / s;
+  auto quot = [&](float x) {
+    if (fast) {
+      const float q0 = x * y;
+      const float r = __builtin_fmaf(-s, q0, x);
+      return __builtin_fmaf(r, y, q0);
+    }
+    return x / s;
+  };
   unsigned char* qr = q + row * static_cast<int64_t>(K);
   for (int k = lane * 16; k < K; k += kWave * 16) {
     const vec8 v0 = *reinterpret_cast<const vec8*>(xr + k);
@@ -59,8 +75,8 @@ __global__ __launch_bounds__(kQuantThreads) void quant_rows_kernel(const T* __re
     float f[16];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      f[i] = fminf(fmaxf(static_cast<float>(v0[i]) / s, -448.f), 448.f);
-      f[8 + i] = fminf(fmaxf(static_cast<float>(v1[i]) / s, -448.f), 448.f);
+      f[i] = fminf(fmaxf(quot(static_cast<float>(v0[i])), -448.f), 448.f);
+      f[8 + i] = fminf(fmaxf(quot(static_cast<float>(v1[i])), -448.f), 448.f);
     }
     u32x4_t o;
     o.x = pack4(f[0], f[1], f[2], f[3]);
