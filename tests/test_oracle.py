@@ -270,3 +270,48 @@ def test_quant_rows_and_fp8_layer_close_to_fp32():
     out32 = oracle.fused_moe(x, w1, w2, logits, 2)
     rel = (out8 - out32).norm() / out32.norm()
     assert rel < 0.08
+
+
+def test_reciprocal_fma_quotient_is_correctly_rounded():
+    """The fp8 row quantisation divides by the row scale with y = RN(1/s), q = RN(x*y),
+    r = RN(x - s*q) (one FMA), RN(q + r*y) (another) for rows whose max|x| lies in [2^-40, 2^40].
+    Exact rational arithmetic: for bf16/fp16 values x with |x| >= 2^-70 (smaller ones encode as
+    zero whatever their last bit) the result is the correctly rounded fp32 quotient x/s."""
+    from fractions import Fraction as F
+    rng = np.random.default_rng(5)
+
+    def rn32(fr):
+        c = np.float32(float(fr))
+        best = None
+        for cand in (np.nextafter(c, np.float32(-np.inf)), c, np.nextafter(c, np.float32(np.inf))):
+            key = (abs(F(float(cand)) - fr), int(np.float32(cand).view(np.uint32)) & 1)
+            if best is None or key < best[0]:
+                best = (key, np.float32(cand))
+        return best[1]
+
+    def grid(n, kind):
+        if kind == "bf16":
+            v = (rng.integers(0, 1 << 16, n, dtype=np.uint32) << 16).view(np.float32)
+        else:
+            v = rng.integers(0, 1 << 16, n, dtype=np.uint16).view(np.float16).astype(np.float32)
+        return v[np.isfinite(v)]
+
+    checked = 0
+    for kind in ("bf16", "f16"):
+        xs = grid(60000, kind)
+        xs = xs[np.abs(xs) >= 2.0 ** -70]
+        am = np.abs(grid(60000, kind))
+        am = am[(am >= 2.0 ** -40) & (am <= 2.0 ** 40)]
+        for x, a in list(zip(xs, am))[:6000]:
+            if abs(x) > a:
+                x, a = np.float32(np.copysign(a, x)), np.float32(abs(x))
+                if not (2.0 ** -40 <= a <= 2.0 ** 40):
+                    continue
+            s = rn32(F(float(a)) / 448)
+            y = rn32(1 / F(float(s)))
+            q = rn32(F(float(x)) * F(float(y)))
+            r = rn32(F(float(x)) - F(float(s)) * F(float(q)))
+            got = rn32(F(float(q)) + F(float(r)) * F(float(y)))
+            assert got.view(np.uint32) == rn32(F(float(x)) / F(float(s))).view(np.uint32), (kind, x, a)
+            checked += 1
+    assert checked > 8000
