@@ -251,6 +251,49 @@ def test_last_round_of_tiles_split_along_k(native, case):
     assert ((out0 - out1).abs() <= 2.0 ** -6 * out0.abs().max()).all()
 
 
+@pytest.mark.parametrize("M", [16, 1536])
+def test_layer_under_graph_capture(native, M):
+    """The whole layer (router logits form) captured into a HIP graph after one warm-up call and
+    replayed three times, with eager work and synchronisations between the replays and new inputs
+    written into the captured buffers: every replay equals the eager result bit for bit.  M=16
+    takes the decode kernels and the fused route+align launch, M=1536 the persistent kernels with
+    their split last round and fix-up launches."""
+    from fast_route_amd import _native as N
+    from fast_route_amd.layers.fused_moe import plan
+    _say(f"graph capture M={M}")
+    dtype = torch.bfloat16
+    H, Fd, E, k = 1024, 2048, 4, 2
+    x, logits, w1, w2 = _inputs(M, H, Fd, E, 55, dtype)
+    xd, ld, w1d, w2d = x.cuda(), logits.cuda(), w1.cuda(), w2.cuda()
+    p = plan(M, H, Fd, E, k, dtype)
+    ws = torch.empty(max(p.workspace_bytes, 256), dtype=torch.uint8, device="cuda")
+    out = torch.empty(M, H, dtype=dtype, device="cuda")
+    lib = N.lib()
+
+    def call(stream):
+        N.check(lib.fr_fused_moe(xd.data_ptr(), w1d.data_ptr(), w2d.data_ptr(), ld.data_ptr(), N.FR_F32, M, H, Fd, E, k, 1,
+                                 N.FR_BF16, out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+
+    call(torch.cuda.current_stream().cuda_stream)  # warm-up: per-kernel attributes are set on first use
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        call(torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        gen = torch.Generator().manual_seed(100 + rep)
+        xd.copy_(torch.randn(M, H, generator=gen).to(dtype))
+        ld.copy_(torch.randn(M, E, generator=gen))
+        call(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        eager = out.clone()
+        out.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager result"
+    _assert_close(out, oracle.fused_moe(xd.cpu(), w1, w2, ld.cpu(), k, True), dtype, "graph replay")
+
+
 def test_stable_and_vllm_route_layers(native):
     """Gate-matrix entry points of both reference layers."""
     from fast_route_amd.layers import stable_route, vllm_route
