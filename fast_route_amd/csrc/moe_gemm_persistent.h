@@ -60,8 +60,12 @@ __device__ __forceinline__ XcdSchedule xcd_schedule(int total, int nper, int xcd
 constexpr int kMaxExperts = 1024;  // limit of the routing entry points
 constexpr int kChunkBlocks = 8;    // token blocks per chunk, at most (measured 4 / 8 / 16: 1675 / 1648 / 1640 us at M=4096,
                                    // 8 and 12 best at M=16384)
-// off[e] = first token block of expert e among the nt real blocks (expert_ids ascends), off[E] = nt
+// off[e] = first token block of expert e among the nt real blocks, off[E] = nt; off[kMaxExperts + 1] = 1
+// if expert_ids does not ascend (routing arrays of another producer, legal for the op-level GEMM): then
+// every tile takes the plain row-major walk, since the table describes no partition of the blocks.
+constexpr int kWalkTable = kMaxExperts + 2;
 __device__ __forceinline__ void expert_block_offsets(const GemmArgs& a, int nt, int* off, int tid, int nthreads) {
+  if (tid == 0) off[kMaxExperts + 1] = 0;
   for (int e = tid; e <= a.num_experts; e += nthreads) {
     int lo = 0, hi = nt;
     while (lo < hi) {
@@ -71,10 +75,20 @@ __device__ __forceinline__ void expert_block_offsets(const GemmArgs& a, int nt, 
     }
     off[e] = lo;
   }
+  __syncthreads();
+  for (int b = tid + 1; b < nt; b += nthreads)
+    if (a.expert_ids[b] < a.expert_ids[b - 1]) off[kMaxExperts + 1] = 1;
+  __syncthreads();
 }
 __device__ __forceinline__ void tile_coords(const GemmArgs& a, const int* off, int lin, int& pid_t, int& pid_f,
                                             int& expert) {
   const int F = a.num_f_tiles;
+  if (off[kMaxExperts + 1]) {
+    pid_t = lin / F;
+    pid_f = lin % F;
+    expert = a.expert_ids[pid_t];
+    return;
+  }
   expert = a.expert_ids[lin / F];  // lin / F is one of the expert's blocks: its tiles are [off[e] * F, off[e + 1] * F)
   const int first = off[expert], len = off[expert + 1] - first;
   const int chunks = (len + a.group_t - 1) / a.group_t, base = len / chunks, rem = len - base * chunks;
@@ -164,9 +178,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   const XcdSchedule xs = xcd_schedule(total, nper, xcd, k_all, a.tail_ws != nullptr);
   const int n_units = xs.rounds + (loc < xs.rest * xs.slices ? 1 : 0);
   if (n_units == 0) return;
-  __shared__ int expert_off[kMaxExperts + 1];
+  __shared__ int expert_off[kWalkTable];
   expert_block_offsets(a, nt, expert_off, threadIdx.x, C::NT);
-  __syncthreads();
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wt = wave / C::WF, wf = wave % C::WF;
@@ -429,9 +442,8 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(const GemmArgs a, int n
   const int nt = min(a.npost[0] / BT, a.num_t_blocks);
   const XcdSchedule xs = xcd_schedule(nt * a.num_f_tiles, nper, xcd, a.K / BK, true);
   if (xs.slices < 2 || t >= xs.rest) return;
-  __shared__ int expert_off[kMaxExperts + 1];
+  __shared__ int expert_off[kWalkTable];
   expert_block_offsets(a, nt, expert_off, threadIdx.x, 256);
-  __syncthreads();
   int pid_t, pid_f, expert;
   tile_coords(a, expert_off, xs.base + xs.rounds * nper + t, pid_t, pid_f, expert);
   const float* wsc = nullptr;

@@ -294,6 +294,31 @@ def test_layer_under_graph_capture(native, M):
     _assert_close(out, oracle.fused_moe(xd.cpu(), w1, w2, ld.cpu(), k, True), dtype, "graph replay")
 
 
+@pytest.mark.parametrize("block", [128, 256])
+def test_grouped_gemm_with_blocks_in_any_order(native, block):
+    """The op-level GEMM only needs every block to belong to one expert; routing arrays whose
+    blocks are not in ascending expert order (here: reversed) are legal input.  The persistent
+    kernels walk tiles expert by expert through a table built from an ascending expert_ids and
+    must fall back to a plain walk when it is not."""
+    from fast_route_amd.ops.fused_moe import invoke_fused_moe_kernel, moe_align_block_size
+    _say(f"grouped GEMM, blocks reversed, block={block}")
+    dtype = torch.bfloat16
+    M, H, Fd, E, k = 1200, 512, 768, 6, 2
+    x, logits, w1, w2 = _inputs(M, H, Fd, E, 41, dtype)
+    w, ids = oracle.gating_topk(logits, k)
+    xd, w1d, wd, idd = x.cuda(), w1.cuda(), w.cuda(), ids.cuda()
+    s, e, npost = moe_align_block_size(idd, block, E)
+    nb = int(npost.item()) // block
+    s2, e2 = s.clone(), e.clone()
+    s2[: nb * block] = s[: nb * block].view(nb, block).flip(0).reshape(-1)
+    e2[:nb] = e[:nb].flip(0)
+    cfg = {"BLOCK_SIZE_M": block, "BLOCK_SIZE_N": 64, "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 8}
+    c1 = torch.empty((M, k, 2 * Fd), dtype=dtype, device="cuda")
+    invoke_fused_moe_kernel(xd, w1d, c1, wd, idd, s2, e2, npost, False, k, cfg)
+    torch.cuda.synchronize()
+    _assert_close(c1.view(M * k, -1), oracle.grouped_gemm(x, w1, w, ids, False, k), dtype, "reversed blocks")
+
+
 def test_stable_and_vllm_route_layers(native):
     """Gate-matrix entry points of both reference layers."""
     from fast_route_amd.layers import stable_route, vllm_route
