@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const P* __restrict__ part
 template <typename T> struct Tiles {  // bf16 / fp16
   typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
-  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0> T128P;  // persistent form (down projection)
+  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;  // persistent form; one wavefront per SIMD issues the loads (2-4 % over each its own)
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
   typedef Cfg<32, 128, 128, 1, 4, 16, 2, 3> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
@@ -53,7 +53,7 @@ template <typename T> struct Tiles {  // bf16 / fp16
 template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per two K-steps
   typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
-  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0> T128P;
+  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
   typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
