@@ -516,7 +516,10 @@ int persistent_grid(int* grid_out) {
     if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e == hipSuccess)
       e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, moe_gemm_persistent_kernel<T, C, EPI>, C::NT, C::LDS_BYTES);
-    if (e != hipSuccess) return fail(FR_E_LAUNCH, "persistent GEMM set-up (%d B LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
+    if (e != hipSuccess) {
+      (void)hipGetLastError();  // reported here: not to be found again by the next launch check
+      return fail(FR_E_LAUNCH, "persistent GEMM set-up (%d B LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
+    }
     if (per_cu < 1 || cus < 8) return fail(FR_E_LAUNCH, "persistent GEMM: occupancy %d on %d CUs", per_cu, cus);
     cached[dev] = cus * per_cu / 8 * 8;
   }
