@@ -80,16 +80,12 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
   switch (block) {
     case 256:
       fill(256, TL::T256::BF, TL::T256::BKB);
-      // One workgroup per CU: the persistent form hides each tile's ring fill and drain behind
-      // its neighbour's.  The fp8 fragments leave no registers for the second address set.
-      if constexpr (sizeof(T) == 2) {
-        return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
-      } else if constexpr (EPI != EPI_SILU) {
-        // fp8: no hand-off between tiles; the down projection still gains the split of its last round, the
-        // gate/up GEMM (short K, register-starved epilogue) is 12 % slower in this form and keeps the plain one
-        if (a.long_k) return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
-      }
-      return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
+      // One workgroup per CU: the persistent form hides each tile's ring fill and drain behind its
+      // neighbour's.  fp8 runs it with one fragment buffer (registers for the second address set): 4-5 %
+      // faster for the down projection, but 6 % slower for the gate/up GEMM (short K, register-starved
+      // epilogue: the hand-off K tiles spill), which keeps the plain kernel.
+      if constexpr (sizeof(T) == 1 && EPI == EPI_SILU) return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
+      else return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
     case 128:
       fill(128, TL::T128::BF, TL::T128::BKB);
       // The down projection has few feature tiles and a long K: it gains from the persistent form's

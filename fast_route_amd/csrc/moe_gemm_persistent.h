@@ -150,7 +150,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
   constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, IW = C::IW, NLI = (XI + WI) * IW;
   constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
-  constexpr bool HANDOFF = !E::SCALED;  // the 8-register fp8 fragments leave no room for a second address set
+  constexpr bool SINGLE = E::SCALED;   // one fragment buffer for fp8 (8-register fragments), two otherwise
+  constexpr bool HANDOFF = true;
   static_assert(S >= 2 && C::SPREAD <= 1, "persistent form: ring of at least two slots, refill in one group");
   static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
   static_assert((S - 1) * NLI <= 63, "vmcnt budget");
@@ -293,18 +294,47 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
         wfr[fb_][j][c] = wtl[woff[j] + (kc ^ wkey[j])];                                 \
     }                                                                                   \
   }
-  // One K-step: NM MFMAs; the fragments of the next step are read after the first half; the
-  // refill loads (ISS_: this wavefront issues, set SET) go out one at a time between the MFMAs.
-#define FR_KSTEP(fb_, READ_NEXT, ISS_, SET, tile_, slot_)                                     \
+  // fragment i_ of the token operand / j_ of the weight operand alone, into buffer 0
+#define FR_READ_X1(sl_, ks_, i_)                                                        \
+  {                                                                                     \
+    const u32x4* xt = lds + (sl_) * C::XCH;                                             \
+    _Pragma("unroll") for (int c = 0; c < FC; ++c) {                                    \
+      const int kc = ((ks_) * C::KGROUPS + kgrp) * FC + c;                              \
+      xf[0][i_][c] = xt[xoff[i_] + (kc ^ xkey[i_])];                                    \
+    }                                                                                   \
+  }
+#define FR_READ_W1(sl_, ks_, j_)                                                        \
+  {                                                                                     \
+    const u32x4* wtl = lds + (sl_) * C::WCH;                                            \
+    _Pragma("unroll") for (int c = 0; c < FC; ++c) {                                    \
+      const int kc = ((ks_) * C::KGROUPS + kgrp) * FC + c;                              \
+      wfr[0][j_][c] = wtl[woff[j_] + (kc ^ wkey[j_])];                                  \
+    }                                                                                   \
+  }
+  // One K-step: NM MFMAs, weight tile j outer, token tile i inner.  HAVE_NEXT: the fragments of K-step
+  // NKS of ring slot NSL follow.  With two fragment buffers they are all read after the first half of
+  // the MFMAs into the other buffer.  With one buffer (SINGLE: fp8, whose fragments are twice as
+  // large) each fragment is read again as soon as its last MFMA of this step has been issued - the
+  // weight fragment j after token tile IT-1, the token fragment i during the last weight tile - which
+  // leaves at least IT-1 MFMAs (64 cycles each for fp8) between a read and its first use.
+  // The refill loads (ISS_: this wavefront issues, set SET) go out one at a time between the MFMAs.
+#define FR_KSTEP(fb_, HAVE_NEXT, NSL, NKS, ISS_, SET, tile_, slot_)                           \
   {                                                                                           \
+    const int fbc = SINGLE ? 0 : (fb_);                                                       \
     _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                          \
       const int j = m / C::IT, i = m % C::IT;                                                 \
-      if constexpr (C::TILE == 32) acc[j][i] = E::m32(wfr[fb_][j], xf[fb_][i], acc[j][i]);    \
-      else acc[j][i] = E::m16(wfr[fb_][j], xf[fb_][i], acc[j][i]);                            \
+      if constexpr (C::TILE == 32) acc[j][i] = E::m32(wfr[fbc][j], xf[fbc][i], acc[j][i]);    \
+      else acc[j][i] = E::m16(wfr[fbc][j], xf[fbc][i], acc[j][i]);                            \
       __builtin_amdgcn_sched_barrier(0);                                                      \
-      if (m == RD_AT) {                                                                       \
-        READ_NEXT;                                                                            \
-        __builtin_amdgcn_sched_barrier(0);                                                    \
+      if (HAVE_NEXT) {                                                                        \
+        if constexpr (SINGLE) {                                                               \
+          if (i == C::IT - 1) FR_READ_W1(NSL, NKS, j)                                         \
+          if (j == C::JF - 1) FR_READ_X1(NSL, NKS, i)                                         \
+          if (i == C::IT - 1 || j == C::JF - 1) __builtin_amdgcn_sched_barrier(0);            \
+        } else if (m == RD_AT) {                                                              \
+          FR_READ_FRAGS(NSL, NKS, fbc ^ 1);                                                   \
+          __builtin_amdgcn_sched_barrier(0);                                                  \
+        }                                                                                     \
       }                                                                                       \
       if (ISS_) {                                                                             \
         _Pragma("unroll") for (int r = 0; r < NLI; ++r)                                       \
@@ -324,13 +354,13 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     const int sn = (sl + 1 == S) ? 0 : sl + 1;                                                 \
     _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
       if (ks + 1 < KS) {                                                                       \
-        FR_KSTEP(ks & 1, FR_READ_FRAGS(sl, ks + 1, (ks + 1) & 1), false, A, 0, 0);             \
+        FR_KSTEP(ks & 1, true, sl, ks + 1, false, A, 0, 0);                                    \
       } else if (LAST) {                                                                       \
-        FR_KSTEP(ks & 1, {}, false, A, 0, 0);                                                  \
+        FR_KSTEP(ks & 1, false, 0, 0, false, A, 0, 0);                                         \
       } else {                                                                                 \
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(VMC) : "memory");                  \
         __builtin_amdgcn_s_barrier();                                                          \
-        FR_KSTEP(ks & 1, FR_READ_FRAGS(sn, 0, 0), (ISS_) && (REFILL), SET, rtile_, sl);        \
+        FR_KSTEP(ks & 1, true, sn, 0, (ISS_) && (REFILL), SET, rtile_, sl);                    \
       }                                                                                        \
     }                                                                                          \
     sl = sn;                                                                                   \
@@ -379,8 +409,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     FR_READ_FRAGS(0, 0, 0);                                                                                \
   }
   // Whole pipeline for an issuing (ISS_ = true) or a non-issuing wavefront.  HANDOFF: the ring
-  // passes from unit to unit as described above; without it (fp8: no registers for the second
-  // address set) every unit fills and drains the ring by itself.
+  // passes from unit to unit as described above; without it every unit fills and drains the ring by
+  // itself (kept for tiles whose registers cannot hold the second address set).
 #define FR_PERSIST(ISS_)                                                                                   \
   {                                                                                                        \
     FR_FILL(ISS_)                                                                                          \
@@ -413,6 +443,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #undef FR_TILE
 #undef FR_KTILE
 #undef FR_KSTEP
+#undef FR_READ_W1
+#undef FR_READ_X1
 #undef FR_READ_FRAGS
 #undef FR_ISSUE_ONE
 #undef FR_MAKE_SET
