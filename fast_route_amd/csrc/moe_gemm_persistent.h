@@ -151,7 +151,6 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, IW = C::IW, NLI = (XI + WI) * IW;
   constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
   constexpr bool SINGLE = E::SCALED;   // one fragment buffer for fp8 (8-register fragments), two otherwise
-  constexpr bool HANDOFF = true;
   static_assert(S >= 2 && C::SPREAD <= 1, "persistent form: ring of at least two slots, refill in one group");
   static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
   static_assert((S - 1) * NLI <= 63, "vmcnt budget");
@@ -408,34 +407,20 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     __builtin_amdgcn_s_barrier();                                                                          \
     FR_READ_FRAGS(0, 0, 0);                                                                                \
   }
-  // Whole pipeline for an issuing (ISS_ = true) or a non-issuing wavefront.  HANDOFF: the ring
-  // passes from unit to unit as described above; without it every unit fills and drains the ring by
-  // itself (kept for tiles whose registers cannot hold the second address set).
+  // Whole pipeline for an issuing (ISS_ = true) or a non-issuing wavefront.
 #define FR_PERSIST(ISS_)                                                                                   \
   {                                                                                                        \
     FR_FILL(ISS_)                                                                                          \
     int sl = 0;                                                                                            \
     int unit = 0;                                                                                          \
-    if constexpr (HANDOFF) {                                                                               \
-      for (; unit + 1 < n_units; ++unit) { /* a next unit exists: hand the ring over to it */              \
-        FR_TILE(ISS_, true)                                                                                \
-        pid_t = n_pid_t; pid_f = n_pid_f; expert = n_expert; xrsA = xrsB; wrsA = wrsB;                     \
-        kb = n_kb; kn = n_kn; tu = n_tu;                                                                   \
-        _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) xsrcA[ih] = xsrcB[ih];                      \
-        _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) wsrcA[ih] = wsrcB[ih];                      \
-      }                                                                                                    \
-      FR_TILE(ISS_, false)                                                                                 \
-    } else {                                                                                               \
-      for (;;) {                                                                                           \
-        FR_TILE(ISS_, false)                                                                               \
-        if (++unit == n_units) break;                                                                      \
-        FR_UNIT(unit, pid_t, pid_f, expert, kb, kn, tu)                                                    \
-        FR_MAKE_SET(pid_t, pid_f, expert, kb, a.sorted[pid_t * BT + rr], xsrcA, wsrcA, xrsA, wrsA)         \
-        __syncthreads(); /* every wavefront is done with the ring before it is filled again */            \
-        FR_FILL(ISS_)                                                                                      \
-        sl = 0;                                                                                            \
-      }                                                                                                    \
+    for (; unit + 1 < n_units; ++unit) { /* a next unit exists: hand the ring over to it */                \
+      FR_TILE(ISS_, true)                                                                                  \
+      pid_t = n_pid_t; pid_f = n_pid_f; expert = n_expert; xrsA = xrsB; wrsA = wrsB;                       \
+      kb = n_kb; kn = n_kn; tu = n_tu;                                                                     \
+      _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) xsrcA[ih] = xsrcB[ih];                        \
+      _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) wsrcA[ih] = wsrcB[ih];                        \
     }                                                                                                      \
+    FR_TILE(ISS_, false)                                                                                   \
   }
   if (IW == 1 || issuer) FR_PERSIST(true) else FR_PERSIST(false)
 #undef FR_PERSIST
