@@ -127,3 +127,25 @@ def test_route_gate_fused_gemm(native, E, topk, H, dtype):
         assert flips.float().mean() < 0.02
         ok = ~flips.any(dim=1)
         torch.testing.assert_close(w.cpu()[ok], ow[ok], atol=1e-4, rtol=0)
+
+
+@pytest.mark.parametrize("E,topk,H", [(8, 2, 264), (64, 6, 256), (24, 3, 512)])
+def test_route_gate_large_batch(native, E, topk, H):
+    """From 16384 tokens on the kernel takes its unsplit form (64 or 128 tokens per workgroup,
+    every wavefront the whole K range of its own tokens); 16500 tokens leave a ragged last
+    workgroup."""
+    from fast_route_amd.ops.stable_route import fused_route
+    M = 16500
+    _say(f"route_gate large batch E={E} k={topk} H={H}")
+    g = torch.Generator().manual_seed(E * 7 + H)
+    h = (torch.randn(M, H, generator=g) / 4).to(torch.bfloat16)
+    gate = (torch.randn(H, E, generator=g) / 4).to(torch.bfloat16)
+    tw = torch.empty(M, topk, dtype=torch.float32, device="cuda")
+    ti = torch.empty(M, topk, dtype=torch.int32, device="cuda")
+    w, ids = fused_route(h.cuda(), gate.cuda(), topk, tw, ti, True)
+    torch.cuda.synchronize()
+    ow, oid = oracle.gating_topk((h.double() @ gate.double()).float(), topk, True)
+    flips = (ids.cpu() != oid)
+    assert flips.float().mean() < 0.02
+    ok = ~flips.any(dim=1)
+    torch.testing.assert_close(w.cpu()[ok], ow[ok], atol=1e-4, rtol=0)
