@@ -164,15 +164,15 @@ def test_op_level_chain_matches_reference_layer_recipe(native, block):
     _assert_close(out, oracle.moe_experts(x, w1, w2, w, ids), dtype, "op chain")
 
 
-def test_block_256_several_tiles_per_workgroup(native):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_block_256_several_tiles_per_workgroup(native, dtype):
     """With more 256x256 tiles than resident workgroups the 2-byte kernel walks several
     tiles per workgroup, the next tile's first loads issued during the current tile's last
     K tiles: 27 token blocks x 16 feature tiles = 432 tiles for at most 256 workgroups,
     so the grid mixes workgroups with one tile and with two."""
     from fast_route_amd import fused_moe
     from fast_route_amd.ops.fused_moe import invoke_fused_moe_kernel, moe_align_block_size
-    _say("block 256, several tiles per workgroup")
-    dtype = torch.bfloat16
+    _say(f"block 256, several tiles per workgroup, {dtype}")
     M, H, Fd, E, k, block = 3000, 512, 2048, 4, 2, 256
     x, logits, w1, w2 = _inputs(M, H, Fd, E, 33, dtype)
     w, ids = oracle.gating_topk(logits, k)
