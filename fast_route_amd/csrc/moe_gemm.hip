@@ -89,8 +89,9 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       else return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
     case 128:
       fill(128, TL::T128::BF, TL::T128::BKB);
-      // The down projection has few feature tiles and a long K: it gains from the persistent form's
-      // split of the last round; the gate/up GEMM at these sizes streams weights and does not.
+      // The gate/up GEMM always takes the persistent form (its walk by expert fetches each expert's
+      // weights once per chunk of token blocks); the down projection of the layer (few feature tiles,
+      // long K) takes it for the split of the last round, a plain grouped GEMM keeps the plain kernel.
       if constexpr (EPI != EPI_SILU) {
         if (a.long_k) return launch_gemm_persistent<T, typename TL::T128P, EPI>(a, splits, st);
       } else {
@@ -165,7 +166,7 @@ int usable_splits(int split_k, int64_t K, int bk) {
 
 int64_t tail_scratch_bytes(int block, int dtype, int64_t K, int64_t N, bool gateup) {
   // The tiles that run persistently: T256 (both GEMMs for 2-byte operands, the down projection for fp8)
-  // and T128P (down projection).  Same K bytes per tile and same feature tile in all of them.
+  // and T128P (both GEMMs).  Same K bytes per tile and same feature tile in all of them.
   typedef Tiles<bf16_t>::T256 C;
   static_assert(Tiles<bf16_t>::T128P::BF == C::BF && Tiles<bf16_t>::T128P::BKB == C::BKB, "same K tile and feature tile");
   static_assert(Tiles<fp8_t>::T256::BF == C::BF && Tiles<fp8_t>::T256::BKB == C::BKB, "same K tile and feature tile");
