@@ -1,5 +1,6 @@
 // Host side of the grouped expert GEMMs: tile selection, launches, top-k combine.
 #include "moe_gemm_persistent.h"
+#include "moe_gemv.h"
 
 namespace fr {
 
@@ -197,6 +198,11 @@ int gateup_impl(const void* x, const float* x_scale, const void* w1, const float
   a.num_valid = (int)n; a.top_k = topk; a.N = (int)F; a.K = (int)H;
   a.num_experts = E;
   a.tail_ws = tail_ws;
+  if (gateup_rows_fits(M, H, block, elem_bytes(dtype))) {
+    // a handful of tokens: stream the weight rows past the token rows without tiles
+    if (dtype == FR_BF16) return launch_gateup_rows<bf16_t>(a, block, sorted_len / block * block, st);
+    return launch_gateup_rows<f16_t>(a, block, sorted_len / block * block, st);
+  }
   return dispatch_dtype<EPI_SILU>(a, dtype, block, 1, sorted_len / block * block, st);
 }
 

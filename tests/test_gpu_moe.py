@@ -251,6 +251,66 @@ def test_last_round_of_tiles_split_along_k(native, case):
     assert ((out0 - out1).abs() <= 2.0 ** -6 * out0.abs().max()).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,H,E,k", [(1, 4096, 8, 2), (2, 4096, 8, 2), (3, 4096, 8, 2), (4, 4096, 8, 2), (4, 8192, 4, 2),
+                                      (2, 4096, 16, 6), (1, 8192, 8, 8)])
+def test_decode_gate_up_by_rows(native, M, H, E, k, dtype):
+    """Up to four tokens with H a multiple of 4096: the gate/up projection streams each weight row
+    past the routing block's token rows (dot products, no tiles) and leaves the same activation
+    layout to the down projection.  H = 8192 with four tokens fills the token-row buffer."""
+    from fast_route_amd import fused_moe
+    _say(f"decode rows M={M} H={H} E={E} k={k} {dtype}")
+    x, logits, w1, w2 = _inputs(M, H, 384, E, 100 + M + k, dtype)
+    out = fused_moe(x.cuda(), w1.cuda(), w2.cuda(), logits.cuda(), k, True)
+    torch.cuda.synchronize()
+    _assert_close(out, oracle.fused_moe(x, w1, w2, logits, k, True), dtype, f"rows M={M} H={H}")
+
+
+@pytest.mark.parametrize("block", [16, 32, 64, 128])
+def test_decode_gate_up_by_rows_matches_tiles(native, block):
+    """The same three tokens through the gate/up entry point with H = 4096 (rows, for blocks up to
+    64 slots; 128-slot blocks keep the tiles) and, zero-extended to H = 4224 (not a multiple of
+    4096: tiles), give the same activations up to the summation order; an expert chosen twice by
+    one token puts more rows into a block than there are tokens, which costs the row form a second
+    pass over that block."""
+    from fast_route_amd import _native as N
+    from fast_route_amd.ops.fused_moe import moe_align_block_size
+    _say(f"decode rows vs tiles block={block}")
+    dtype = torch.bfloat16
+    M, H, Fd, E, k = 3, 4096, 256, 4, 2
+    g = torch.Generator().manual_seed(block)
+    x = torch.randn(M, H, generator=g).to(dtype)
+    w1 = (torch.randn(E, 2 * Fd, H, generator=g) * 0.02).to(dtype)
+    ids = torch.tensor([[1, 1], [1, 3], [0, 1]], dtype=torch.int32)   # expert 1: 4 rows from 3 tokens
+    lib, st = N.lib(), torch.cuda.current_stream().cuda_stream
+    s, e, npost = moe_align_block_size(ids.cuda(), block, E)
+    acts = []
+    for pad in (0, 128):
+        xd = torch.nn.functional.pad(x, (0, pad)).contiguous().cuda()
+        w1d = torch.nn.functional.pad(w1, (0, pad)).contiguous().cuda()
+        act = torch.zeros(s.numel(), Fd, dtype=dtype, device="cuda")
+        N.check(lib.fr_moe_gateup_silu(xd.data_ptr(), w1d.data_ptr(), s.data_ptr(), e.data_ptr(), npost.data_ptr(), M,
+                                       H + pad, Fd, E, k, block, N.FR_BF16, act.data_ptr(), None, st))
+        torch.cuda.synchronize()
+        acts.append(act.float().cpu())
+    # reference: every real slot's row (the tile kernel also fills the padding slots of a block, with
+    # values nobody reads; the row form leaves them alone)
+    sc = s.cpu()
+    ref = torch.zeros_like(acts[0])
+    real = torch.zeros(ref.shape[0], dtype=torch.bool)
+    for slot in range(int(npost.item())):
+        sid = int(sc[slot])
+        if sid < M * k:
+            gu = x[sid // k].float() @ w1[int(ids.view(-1)[sid])].float().T
+            ref[slot] = torch.nn.functional.silu(gu[:Fd]) * gu[Fd:]
+            real[slot] = True
+    assert int(real.sum()) == M * k
+    for a in acts:
+        assert ((a - ref).abs() <= 2.0 ** -7 * ref.abs() + 1e-3)[real].all()
+    if block <= 64:
+        assert acts[0][~real].abs().sum() == 0
+
+
 @pytest.mark.parametrize("M", [16, 1536])
 def test_layer_under_graph_capture(native, M):
     """The whole layer (router logits form) captured into a HIP graph after one warm-up call and
