@@ -202,8 +202,15 @@ def kernel_roofline(shape, rec, fp8=False):
     eb = 1 if fp8 else 2
     byts = rec["active_experts"] * 2 * F * H * eb + M * H * eb + M * topk * F * 2
     peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
-    # 256-row routing blocks of 2-byte operands run the persistent form of the kernel
-    name = ("moe_gemm_persistent_kernel" if rec["block"] == 256 and not fp8 else "moe_gemm_kernel") + "<EPI_SILU>"
+    # which kernel the library picks for the gate/up GEMM: weight rows against token rows for up to 4
+    # tokens of 2-byte operands with H a multiple of 4096, the persistent tile kernel for 128-row blocks
+    # and for 256-row blocks of 2-byte operands, the plain tile kernel otherwise
+    if not fp8 and M <= 4 and H % 4096 == 0 and M * H * 2 <= 65536:
+        name = "gateup_rows_kernel"
+    elif rec["block"] == 128 or (rec["block"] == 256 and not fp8):
+        name = "moe_gemm_persistent_kernel<EPI_SILU>"
+    else:
+        name = "moe_gemm_kernel<EPI_SILU>"
     if flops / (peak * 1e12) >= byts / (PEAK_HBM_GBS * 1e9):
         ach = flops / dur / 1e12
         return {"kernel": name, "bound": "mfma", "achieved": round(ach, 2), "peak": peak,
