@@ -311,18 +311,19 @@ def test_decode_gate_up_by_rows_matches_tiles(native, block):
         assert acts[0][~real].abs().sum() == 0
 
 
-@pytest.mark.parametrize("M", [16, 1536])
+@pytest.mark.parametrize("M", [2, 16, 1536])
 def test_layer_under_graph_capture(native, M):
     """The whole layer (router logits form) captured into a HIP graph after one warm-up call and
     replayed three times, with eager work and synchronisations between the replays and new inputs
-    written into the captured buffers: every replay equals the eager result bit for bit.  M=16
+    written into the captured buffers: every replay equals the eager result bit for bit.  M=2
+    (with H = 4096) takes the gate/up projection by weight rows, M=16
     takes the decode kernels and the fused route+align launch, M=1536 the persistent kernels with
     their split last round and fix-up launches."""
     from fast_route_amd import _native as N
     from fast_route_amd.layers.fused_moe import plan
     _say(f"graph capture M={M}")
     dtype = torch.bfloat16
-    H, Fd, E, k = 1024, 2048, 4, 2
+    H, Fd, E, k = (4096, 512, 4, 2) if M == 2 else (1024, 2048, 4, 2)
     x, logits, w1, w2 = _inputs(M, H, Fd, E, 55, dtype)
     xd, ld, w1d, w2d = x.cuda(), logits.cuda(), w1.cuda(), w2.cuda()
     p = plan(M, H, Fd, E, k, dtype)
