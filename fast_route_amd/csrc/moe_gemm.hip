@@ -198,7 +198,7 @@ int gateup_impl(const void* x, const float* x_scale, const void* w1, const float
   a.num_valid = (int)n; a.top_k = topk; a.N = (int)F; a.K = (int)H;
   a.num_experts = E;
   a.tail_ws = tail_ws;
-  if (gateup_rows_fits(M, H, block, elem_bytes(dtype))) {
+  if (gateup_rows_fits(M, H, block, sorted_len, elem_bytes(dtype))) {
     // a handful of tokens: stream the weight rows past the token rows without tiles
     if (dtype == FR_BF16) return launch_gateup_rows<bf16_t>(a, block, sorted_len / block * block, st);
     return launch_gateup_rows<f16_t>(a, block, sorted_len / block * block, st);

@@ -129,9 +129,10 @@ __global__ void __launch_bounds__(kRowsThreads) gateup_rows_kernel(GemmArgs a, i
 
 // Whether the row form takes this gate/up projection: 2-byte operands, at most kRowsMax tokens,
 // routing blocks of at most 64 slots, weight rows of whole rounds, token rows that fit the LDS.
-inline bool gateup_rows_fits(int64_t M, int64_t K, int block, int elem_bytes) {
+inline bool gateup_rows_fits(int64_t M, int64_t K, int block, int64_t sorted_len, int elem_bytes) {
   const int64_t rows = M < block ? M : block;
-  return elem_bytes == 2 && M >= 1 && M <= kRowsMax && block <= kWave && K % kRowsK == 0 && rows * K * 2 <= kRowsLds;
+  return elem_bytes == 2 && M >= 1 && M <= kRowsMax && block <= kWave && K % kRowsK == 0 && rows * K * 2 <= kRowsLds &&
+         sorted_len / block <= 65535;  // routing blocks are the grid's y dimension
 }
 
 template <typename T>
