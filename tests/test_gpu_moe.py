@@ -139,6 +139,22 @@ def test_layer_rejects_bad_arguments(native):
         fused_moe(x.cuda(), w1.cuda(), w2.cuda(), logits.cuda(), 9)  # topk > E
 
 
+def test_layer_with_64_row_blocks(native):
+    """26 to 52 pairs per expert with H >= 4096: the plan takes 64-row routing blocks (one block per
+    expert, K of the down projection cut into slices)."""
+    from fast_route_amd import fused_moe
+    from fast_route_amd.layers.fused_moe import plan
+    _say("layer with 64-row blocks")
+    dtype = torch.bfloat16
+    M, H, Fd, E, k = 160, 4096, 1024, 8, 2
+    p = plan(M, H, Fd, E, k, dtype)
+    assert p.block == 64 and p.split_k >= 2
+    x, logits, w1, w2 = _inputs(M, H, Fd, E, 64, dtype)
+    out = fused_moe(x.cuda(), w1.cuda(), w2.cuda(), logits.cuda(), k, True)
+    torch.cuda.synchronize()
+    _assert_close(out, oracle.fused_moe(x, w1, w2, logits, k, True), dtype, "64-row blocks")
+
+
 @pytest.mark.parametrize("block", [16, 32, 64, 128, 256])
 def test_op_level_chain_matches_reference_layer_recipe(native, block):
     """The reference layer spelled with its own ops (layers/stable_route.py:82-102):
