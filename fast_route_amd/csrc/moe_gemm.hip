@@ -35,8 +35,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const P* __restrict__ part
 // the 16-row block); every block except 64 streams tiles HBM -> LDS directly.
 //   256 / 128 rows: 8 wavefronts, 32x32 MFMA, 2- or 3-slot ring (compute-bound regime);
 //                   in the 256-row tile one wavefront per SIMD issues the loads of both;
-//   64 rows:        8 wavefronts, register-staged double buffer (op-level API only;
-//                   the fused layer goes from 32-row to 128-row blocks);
+//   64 rows:        3-slot ring, 8 wavefronts (4 with 256-byte row segments for the gate/up GEMM);
+//                   fp8 keeps the register-staged double buffer (op-level API only there);
 //   32 / 16 rows:   decode regime, 16x16 MFMA, 3-slot ring, two workgroups per CU:
 //                   weight streaming at HBM rate.  The gate/up GEMM (short weight rows
 //                   of H elements, many of them) streams faster with 512-byte row
@@ -45,7 +45,8 @@ template <typename T> struct Tiles {  // bf16 / fp16
   typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;  // persistent form; one wavefront per SIMD issues the loads (2-4 % over each its own)
-  typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
+  typedef Cfg<64, 256, 128, 2, 4, 32, 1, 3, 3> T64;    // 3-slot ring like the 128-row tile (5 % over the register-staged form)
+  typedef Cfg<64, 128, 256, 2, 2, 32, 1, 3> T64U;      // gate/up: 256-byte row segments, 4 wavefronts (another 5 %)
   typedef Cfg<32, 128, 128, 1, 4, 16, 2, 3> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
   typedef Cfg<32, 128, 512, 1, 4, 16, 1, 2> T32L;
@@ -56,6 +57,7 @@ template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
+  typedef T64 T64U;
   typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
   typedef Cfg<32, 128, 512, 1, 4, 16, 1, 2> T32L;
@@ -99,7 +101,13 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
         return launch_gemm_persistent<T, typename TL::T128P, EPI>(a, splits, st);
       }
       return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
-    case 64: fill(64, TL::T64::BF, TL::T64::BKB); return launch_gemm<T, typename TL::T64, EPI>(a, splits, st);
+    case 64:
+      if (EPI == EPI_SILU && a.K % (TL::T64U::BKB / static_cast<int>(sizeof(T))) == 0) {
+        fill(64, TL::T64U::BF, TL::T64U::BKB);
+        return launch_gemm<T, typename TL::T64U, EPI>(a, splits, st);
+      }
+      fill(64, TL::T64::BF, TL::T64::BKB);
+      return launch_gemm<T, typename TL::T64, EPI>(a, splits, st);
     case 32:
       if (EPI == EPI_SILU && a.K % (TL::T32L::BKB / static_cast<int>(sizeof(T))) == 0) {
         fill(32, TL::T32L::BF, TL::T32L::BKB);
