@@ -139,13 +139,13 @@ def test_layer_rejects_bad_arguments(native):
         fused_moe(x.cuda(), w1.cuda(), w2.cuda(), logits.cuda(), 9)  # topk > E
 
 
-def test_layer_with_64_row_blocks(native):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_layer_with_64_row_blocks(native, dtype):
     """26 to 52 pairs per expert with H >= 4096: the plan takes 64-row routing blocks (one block per
     expert, K of the down projection cut into slices)."""
     from fast_route_amd import fused_moe
     from fast_route_amd.layers.fused_moe import plan
-    _say("layer with 64-row blocks")
-    dtype = torch.bfloat16
+    _say(f"layer with 64-row blocks {dtype}")
     M, H, Fd, E, k = 160, 4096, 1024, 8, 2
     p = plan(M, H, Fd, E, k, dtype)
     assert p.block == 64 and p.split_k >= 2
