@@ -22,6 +22,18 @@ namespace fr {
 
 enum { EPI_PLAIN = 0, EPI_SILU = 1, EPI_DOWN = 2 };
 
+// Cache policy bits of the weight-tile loads (0 = default, 2 = non-temporal).  Tiles of up to 64 token
+// rows stream every weight byte once (one or two blocks per expert): marked non-temporal the stream does
+// not displace the token rows and its own neighbours in L2, and the 16-row gate/up GEMM goes from 6.5 to
+// 6.9 TB/s, the down projection from 5.96 to 6.65 TB/s.  The larger tiles re-read weight tiles from L2
+// for the other token blocks of an expert and keep the default (non-temporal: +1.5 % at M = 1024).
+#ifndef FR_W_AUX
+#define FR_W_AUX (C::BT <= 64 ? 2 : 0)
+#endif
+#ifndef FR_W_AUXP
+#define FR_W_AUXP 0
+#endif
+
 struct GemmArgs {
   const void* X;        // token rows [*, K]
   int64_t ldx;          // row stride of X in elements
@@ -489,7 +501,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     if ((q_) < WI * IW) {                                                                                  \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
           wrs, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vw_) * (kWave * 16)), \
-          16, wsrc[(q_) < WI * IW ? (q_) : 0], (tile_) * C::BKB, 0, 0);                                    \
+          16, wsrc[(q_) < WI * IW ? (q_) : 0], (tile_) * C::BKB, 0, FR_W_AUX);                                    \
     } else {                                                                                               \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
           xrs, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WI * IW) / IW) * NW + vw_) * (kWave * 16)), \
