@@ -26,12 +26,10 @@ enum { EPI_PLAIN = 0, EPI_SILU = 1, EPI_DOWN = 2 };
 // rows stream every weight byte once (one or two blocks per expert): marked non-temporal the stream does
 // not displace the token rows and its own neighbours in L2, and the 16-row gate/up GEMM goes from 6.5 to
 // 6.9 TB/s, the down projection from 5.96 to 6.65 TB/s.  The larger tiles re-read weight tiles from L2
-// for the other token blocks of an expert and keep the default (non-temporal: +1.5 % at M = 1024).
+// for the other token blocks of an expert and keep the default (non-temporal in the persistent 128-row
+// kernel: -2 % at M = 224..384 with one block per expert, +14 % at M = 512 on 8 experts).
 #ifndef FR_W_AUX
 #define FR_W_AUX (C::BT <= 64 ? 2 : 0)
-#endif
-#ifndef FR_W_AUXP
-#define FR_W_AUXP 0
 #endif
 
 struct GemmArgs {

@@ -274,7 +274,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     if ((q_) < WI * IW) {                                                                                   \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
           wrs##SET, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vwi_) * (kWave * 16)), \
-          16, wsrc##SET[(q_) < WI * IW ? (q_) : 0], (tile_) * C::BKB, 0, FR_W_AUXP);                        \
+          16, wsrc##SET[(q_) < WI * IW ? (q_) : 0], (tile_) * C::BKB, 0, 0);                                \
     } else {                                                                                                \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
           xrs##SET, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WI * IW) / IW) * NW + vwi_) * (kWave * 16)), \
