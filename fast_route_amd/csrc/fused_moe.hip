@@ -87,12 +87,11 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // Between 26 and 52 pairs per expert with a long gate/up K the 64-row tile wins: one block per expert
   // where 32-row blocks stream every expert's weights through the CUs twice, and half the MFMA and LDS work
   // of the 128-row tile (measured at H = 4096, F = 14336, E = 8: M = 112..192 4-6 % faster than either;
-  // at H = 2048, F = 1408, E = 64 with skewed load it is slower than the 128-row tile, hence the K condition;
-  // fp8 not measured: it keeps 32- and 128-row blocks).
+  // at H = 2048, F = 1408, E = 64 with skewed load it is slower than the 128-row tile, hence the K condition).
   int block;
   if (avg <= 8) block = 16;
-  else if (avg < 26 || (avg < 32 && (H < 4096 || dtype == FR_FP8_E4M3))) block = 32;
-  else if (avg < 52 && H >= 4096 && dtype != FR_FP8_E4M3) block = 64;
+  else if (avg < 26 || (avg < 32 && H < 4096)) block = 32;
+  else if (avg < 52 && H >= 4096) block = 64;
   else if (avg < t256) block = 128;
   else block = 256;
   // Down projection: N = H gives few feature tiles, so K is split.

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const P* __restrict__ part
 //   256 / 128 rows: 8 wavefronts, 32x32 MFMA, 2- or 3-slot ring (compute-bound regime);
 //                   in the 256-row tile one wavefront per SIMD issues the loads of both;
 //   64 rows:        3-slot ring, 8 wavefronts (4 with 256-byte row segments for the gate/up GEMM);
-//                   fp8 keeps the register-staged double buffer (op-level API only there);
+//                   (the register-staged double buffer of STAGES == 0 is no longer used by any tile);
 //   32 / 16 rows:   decode regime, 16x16 MFMA, 3-slot ring, two workgroups per CU:
 //                   weight streaming at HBM rate.  The gate/up GEMM (short weight rows
 //                   of H elements, many of them) streams faster with 512-byte row
@@ -56,8 +56,8 @@ template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per
   typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;
-  typedef Cfg<64, 256, 128, 2, 4, 32, 1, 0> T64;
-  typedef T64 T64U;
+  typedef Cfg<64, 256, 128, 2, 4, 32, 1, 3, 3> T64;
+  typedef Cfg<64, 128, 256, 2, 2, 32, 1, 3> T64U;
   typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;
   typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
   typedef Cfg<32, 128, 512, 1, 4, 16, 1, 2> T32L;

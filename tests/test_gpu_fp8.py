@@ -66,8 +66,28 @@ def test_fp8_layer_vs_oracle(native, M):
     assert (o - full).norm() / full.norm() < 0.08
 
 
+def test_fp8_layer_with_64_row_blocks(native):
+    """H = 4096 with 40 pairs per expert: the plan takes 64-row routing blocks for fp8 too."""
+    from fast_route_amd import fused_moe_fp8, prepare_weights_fp8
+    from fast_route_amd.layers.fused_moe import plan
+    _say("fp8 layer with 64-row blocks")
+    M, H, Fd, E, k = 160, 4096, 1024, 8, 2
+    from fast_route_amd import _native as N
+    assert plan(M, H, Fd, E, k, None, code=N.FR_FP8_E4M3).block == 64
+    x, logits, w1, w2 = oracle.make_inputs(M, H, Fd, E, seed=64)
+    x, w1, w2 = x.bfloat16(), w1.bfloat16(), w2.bfloat16()
+    w1q, w1s, w2q, w2s = prepare_weights_fp8(w1.cuda(), w2.cuda())
+    out = fused_moe_fp8(x.cuda(), w1q, w1s, w2q, w2s, logits.cuda(), k, True)
+    torch.cuda.synchronize()
+    ref, _ = oracle.fused_moe_fp8(x, w1, w2, logits, k, True)
+    o = out.float().cpu()
+    assert torch.isfinite(o).all()
+    assert (o - ref).norm() / ref.norm() <= 1e-2
+    assert (o - ref).abs().max() <= 2.0 ** -5 * ref.abs().max()
+
+
 def test_fp8_mixtral_shape_sampled(native):
-    """Full fp8 workload shape (H4096 F14336 E8 top2), M in {16, 256, 4096}: sampled tokens vs the
+    """Full fp8 workload shape (H4096 F14336 E8 top2), M in {16, 128, 256, 4096}: sampled tokens vs the
     oracle.  At M=4096 the down projection runs the persistent form with its last round of tiles
     split along K."""
     from fast_route_amd import fused_moe_fp8, prepare_weights_fp8
@@ -77,7 +97,7 @@ def test_fp8_mixtral_shape_sampled(native):
     w2 = (torch.randn(E, H, Fd, generator=g, device="cuda") * 0.02).bfloat16()
     w1q, w1s, w2q, w2s = prepare_weights_fp8(w1, w2)
     w1c, w2c = w1.cpu(), w2.cpu()
-    for M in (16, 256, 4096):
+    for M in (16, 128, 256, 4096):
         _say(f"fp8 mixtral M={M}")
         x = torch.randn(M, H, generator=g, device="cuda").bfloat16()
         logits = torch.randn(M, E, generator=g, device="cuda")
