@@ -109,8 +109,10 @@ typedef struct fr_moe_plan {
 int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk, int dtype, fr_moe_plan* plan);
 
 /* act[s, :] = silu(x[t] @ W1[e, :F]^T) * (x[t] @ W1[e, F:]^T) for every sorted
- * slot s < num_tokens_post_pad (t = sorted_token_ids[s] / topk, padding slots
- * compute on token 0), written at row s of act[sorted_len, F].
+ * slot s < num_tokens_post_pad that holds a pair (t = sorted_token_ids[s] / topk),
+ * written at row s of act[sorted_len, F].  Rows of padding slots are unspecified
+ * (the tile kernels fill them from token 0, the decode form for up to 4 tokens
+ * leaves them untouched); nothing downstream reads them.
  * Replaces: grouped GEMM 1 + silu_and_mul,
  * fast_route/fast_route/layers/stable_route.py:85-90.
  * `tail_ws`: NULL, or 256-byte aligned device scratch of plan.tail_bytes.  With
