@@ -9,6 +9,7 @@ evaluated on the same rounded operands we require
 """
 import sys
 
+import numpy as np
 import pytest
 import torch
 
@@ -497,3 +498,23 @@ def test_mixtral_shape_sampled_tokens_and_properties(native):
         a = fused_experts(x, w1, w2, w, ids)
         b = fused_experts(x, w1, w2, 2 * w, ids)
         assert torch.equal(a, out) and torch.equal(b.float(), 2 * a.float())
+
+
+def test_random_shapes_against_oracle(native):
+    """Forty seeded random layer shapes (token count, widths, expert count, top-k, dtype, renormalisation)
+    against the oracle: every plan boundary gets neighbours on both sides sooner or later."""
+    from fast_route_amd import fused_moe
+    rng = np.random.default_rng(20240607)
+    for case in range(40):
+        E = int(rng.choice([1, 2, 3, 4, 8, 16, 60, 64]))
+        k = int(rng.integers(1, min(E, 8) + 1))
+        H = int(rng.choice([128, 256, 384, 512, 1024, 4096]))
+        Fd = int(rng.choice([128, 256, 384, 640]))
+        M = int(rng.choice([1, 2, 3, 4, 5, 7, 17, 33, 100, 257, 600]) if rng.random() < 0.7 else rng.integers(1, 700))
+        dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
+        renorm = bool(rng.random() < 0.7)
+        _say(f"random case {case}: M={M} H={H} F={Fd} E={E} k={k} {dtype} renorm={renorm}")
+        x, logits, w1, w2 = _inputs(M, H, Fd, E, 1000 + case, dtype, zipf=bool(rng.random() < 0.3))
+        out = fused_moe(x.cuda(), w1.cuda(), w2.cuda(), logits.cuda(), k, renorm)
+        torch.cuda.synchronize()
+        _assert_close(out, oracle.fused_moe(x, w1, w2, logits, k, renorm), dtype, f"random case {case}")
