@@ -137,3 +137,26 @@ def test_fp8_down_projection_tail_split(native):
     assert torch.isfinite(o).all()
     assert (o - ref).norm() / ref.norm() <= 1e-2
     assert (o - ref).abs().max() <= 2.0 ** -5 * ref.abs().max()
+
+
+def test_fp8_random_shapes_against_oracle(native):
+    """Sixteen seeded random fp8 layer shapes against the oracle (same tolerance as above)."""
+    from fast_route_amd import fused_moe_fp8, prepare_weights_fp8
+    rng = np.random.default_rng(8)
+    for case in range(16):
+        E = int(rng.choice([1, 2, 4, 8, 16, 64]))
+        k = int(rng.integers(1, min(E, 6) + 1))
+        H = int(rng.choice([256, 512, 1024, 4096]))
+        Fd = int(rng.choice([256, 512, 768]))
+        M = int(rng.choice([1, 2, 5, 17, 40, 100, 160, 257, 500]))
+        _say(f"fp8 random case {case}: M={M} H={H} F={Fd} E={E} k={k}")
+        x, logits, w1, w2 = oracle.make_inputs(M, H, Fd, E, seed=500 + case)
+        x, w1, w2 = x.bfloat16(), w1.bfloat16(), w2.bfloat16()
+        w1q, w1s, w2q, w2s = prepare_weights_fp8(w1.cuda(), w2.cuda())
+        out = fused_moe_fp8(x.cuda(), w1q, w1s, w2q, w2s, logits.cuda(), k, True)
+        torch.cuda.synchronize()
+        ref, _ = oracle.fused_moe_fp8(x, w1, w2, logits, k, True)
+        o = out.float().cpu()
+        assert torch.isfinite(o).all()
+        assert (o - ref).norm() / ref.norm() <= 1e-2, f"case {case}"
+        assert (o - ref).abs().max() <= 2.0 ** -5 * ref.abs().max(), f"case {case}"
