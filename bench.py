@@ -29,6 +29,7 @@ SHAPES = {
     "mixtral": dict(H=4096, F=14336, E=8, topk=2, zipf=False, sweep=[1, 16, 64, 256, 1024, 4096, 16384]),
     "fine": dict(H=2048, F=1408, E=64, topk=6, zipf=True, sweep=[1, 32, 128, 512, 2048, 8192]),
     "small": dict(H=1024, F=3584, E=8, topk=2, zipf=False, sweep=[64]),
+    "mixtral22b": dict(H=6144, F=16384, E=8, topk=2, zipf=False, sweep=[1, 16, 128, 1024, 4096]),
 }
 
 
@@ -203,9 +204,9 @@ def kernel_roofline(shape, rec, fp8=False):
     byts = rec["active_experts"] * 2 * F * H * eb + M * H * eb + M * topk * F * 2
     peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
     # which kernel the library picks for the gate/up GEMM: weight rows against token rows for up to 4
-    # tokens of 2-byte operands with H a multiple of 4096, the persistent tile kernel for 128-row blocks
+    # tokens of 2-byte operands with H = 4096, 5120, 6144, 7168 or 8192, the persistent tile kernel for 128-row blocks
     # and for 256-row blocks of 2-byte operands, the plain tile kernel otherwise
-    if not fp8 and M <= 4 and H % 4096 == 0 and M * H * 2 <= 65536:
+    if not fp8 and M <= 4 and H >= 4096 and H % 512 == 0 and any(H // 512 % c == 0 for c in (5, 6, 7, 8)) and M * H * 2 <= 65536:
         name = "gateup_rows_kernel"
     elif rec["block"] == 128 or (rec["block"] == 256 and not fp8):
         name = "moe_gemm_persistent_kernel<EPI_SILU>"

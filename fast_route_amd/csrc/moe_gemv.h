@@ -20,8 +20,7 @@ namespace fr {
 
 constexpr int kRowsMax = 4;        // tokens in the batch (hence token rows per pass over a routing block) the row form takes
 constexpr int kRowsThreads = 256;  // 4 wavefronts
-constexpr int kRowsChunks = 8;     // 16-byte loads per lane, row and round
-constexpr int kRowsK = kRowsChunks * kWave * 8;  // elements of a row per round: 4096
+constexpr int kRowsMinK = 4096;    // shorter rows: the tile kernel is as fast (measured at 1024 and 2048)
 constexpr int kRowsWaves = 4096;   // wavefronts the feature runs are cut for: 16 on each of 256 CUs
 constexpr int kRowsWaveBytes = 7 * 16384;  // weight bytes a wavefront streams
 constexpr int kRowsLds = 65536;    // token rows in LDS: the default dynamic limit
@@ -50,16 +49,14 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-// K is a multiple of kRowsK elements: a lane loads kRowsChunks 16-byte chunks of the gate row and of the
-// up row per round (shorter rows, two features at a time to keep as many loads in flight, ran no faster
-// than the tile kernel: they stay there).
+// CH = 16-byte chunks per lane, row and round: a weight row is `rounds` x CH x 512 elements (CH = 8 for K = 4096
+// and 8192, 5 for 5120, 6 for 6144, 7 for 7168); a lane has 2 * CH loads in flight.
 // grid.x * 4 wavefronts cover the F features in runs of `fpw`; grid.y = routing blocks (upper bound).
 // A block's slots are taken `rows` at a time (rows = tokens in the batch <= kRowsMax): a token
 // selects an expert once, so all rows of a block are in its first pass and the later passes find
 // nothing; ids with repeated experts per token still come out right, at one more pass over the weights.
-template <typename T>
+template <typename T, int CH>
 __global__ void __launch_bounds__(kRowsThreads) gateup_rows_kernel(GemmArgs a, int block, int rows, int fpw) {
-  constexpr int CH = kRowsChunks;
   extern __shared__ u32x4 xs[];  // rows x K/8 chunks
   const int b = blockIdx.y;
   if (b * block >= *a.npost) return;
@@ -127,12 +124,21 @@ __global__ void __launch_bounds__(kRowsThreads) gateup_rows_kernel(GemmArgs a, i
   }
 }
 
+// Chunks per round for rows of K elements: the largest of 8..5 that divides K / 512, or 0.
+inline int rows_chunks(int64_t K) {
+  if (K % 512 != 0) return 0;
+  const int64_t nc = K / 512;
+  for (int ch = 8; ch >= 5; --ch)
+    if (nc % ch == 0) return ch;
+  return 0;
+}
+
 // Whether the row form takes this gate/up projection: 2-byte operands, at most kRowsMax tokens,
 // routing blocks of at most 64 slots, weight rows of whole rounds, token rows that fit the LDS.
 inline bool gateup_rows_fits(int64_t M, int64_t K, int block, int64_t sorted_len, int elem_bytes) {
   const int64_t rows = M < block ? M : block;
-  return elem_bytes == 2 && M >= 1 && M <= kRowsMax && block <= kWave && K % kRowsK == 0 && rows * K * 2 <= kRowsLds &&
-         sorted_len / block <= 65535;  // routing blocks are the grid's y dimension
+  return elem_bytes == 2 && M >= 1 && M <= kRowsMax && block <= kWave && K >= kRowsMinK && rows_chunks(K) != 0 &&
+         rows * K * 2 <= kRowsLds && sorted_len / block <= 65535;  // routing blocks are the grid's y dimension
 }
 
 template <typename T>
@@ -150,7 +156,13 @@ int launch_gateup_rows(const GemmArgs& a, int block, int64_t sorted_len, hipStre
   const dim3 grid(static_cast<unsigned>(ceil_div(a.N, static_cast<int64_t>(kRowsThreads / kWave) * fpw)),
                   static_cast<unsigned>(sorted_len / block));
   const size_t lds = static_cast<size_t>(rows) * a.K * sizeof(T);
-  hipLaunchKernelGGL((gateup_rows_kernel<T>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw);
+  switch (rows_chunks(a.K)) {
+    case 8: hipLaunchKernelGGL((gateup_rows_kernel<T, 8>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw); break;
+    case 7: hipLaunchKernelGGL((gateup_rows_kernel<T, 7>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw); break;
+    case 6: hipLaunchKernelGGL((gateup_rows_kernel<T, 6>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw); break;
+    case 5: hipLaunchKernelGGL((gateup_rows_kernel<T, 5>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw); break;
+    default: return fail(FR_E_SHAPE, "gate/up by rows: K=%d", a.K);
+  }
   return check_launch("gateup_rows_kernel");
 }
 

@@ -270,9 +270,10 @@ def test_last_round_of_tiles_split_along_k(native, case):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,H,E,k", [(1, 4096, 8, 2), (2, 4096, 8, 2), (3, 4096, 8, 2), (4, 4096, 8, 2), (4, 8192, 4, 2),
-                                      (2, 4096, 16, 6), (1, 8192, 8, 8)])
+                                      (2, 4096, 16, 6), (1, 8192, 8, 8), (3, 5120, 4, 2), (2, 6144, 8, 2), (4, 7168, 4, 3)])
 def test_decode_gate_up_by_rows(native, M, H, E, k, dtype):
-    """Up to four tokens with H a multiple of 4096: the gate/up projection streams each weight row
+    """Up to four tokens with H = 4096, 5120, 6144, 7168 or 8192 (rows of 5 to 8 rounds' chunks): the gate/up
+    projection streams each weight row
     past the routing block's token rows (dot products, no tiles) and leaves the same activation
     layout to the down projection.  H = 8192 with four tokens fills the token-row buffer."""
     from fast_route_amd import fused_moe
