@@ -318,7 +318,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   // leaves at least IT-1 MFMAs (64 cycles each for fp8) between a read and its first use.
   // The refill loads (ISS_: this wavefront issues, set SET) go out one at a time between the MFMAs.
 #define FR_KSTEP(fb_, HAVE_NEXT, NSL, NKS, ISS_, SET, tile_, slot_)                           \
-  {                                                                                           \
+  if (on_) {                                                                                  \
     const int fbc = SINGLE ? 0 : (fb_);                                                       \
     _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                          \
       const int j = m / C::IT, i = m % C::IT;                                                 \
@@ -370,6 +370,18 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   // refill the ring during the last S K tiles of this one.
 #define FR_TILE(ISS_, NEXT)                                                                                \
   {                                                                                                        \
+    /* A wavefront that issues no loads and whose token rows of this block are all padding (the upper */   \
+    /* half of a block that holds at most half a block of pairs) has nothing to multiply: it keeps the */  \
+    /* barriers and leaves the MFMA pipe and the LDS to the wavefront it shares the SIMD with.  When */     \
+    /* it has rows again, the fragments its skipped read-ahead would have brought are read here. */         \
+    bool on_ = true;                                                                                       \
+    if (!(ISS_)) {                                                                                         \
+      bool any_ = false;                                                                                   \
+      _Pragma("unroll") for (int r0_ = 0; r0_ < C::TT; r0_ += kWave)                                       \
+        any_ |= a.sorted[pid_t * BT + wt * C::TT + r0_ + lane] < a.num_valid;                              \
+      on_ = __ballot(any_) != 0;                                                                           \
+      if (on_) FR_READ_FRAGS(sl, 0, 0)                                                                     \
+    }                                                                                                      \
     if (NEXT) {                                                                                            \
       FR_UNIT(unit + 1, n_pid_t, n_pid_f, n_expert, n_kb, n_kn, n_tu)                                      \
       if (a.top_k > 0) {                                                                                   \
