@@ -13,7 +13,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libfast_route_hip.so")
-SOURCES = ["fr_error.hip", "gating.hip", "routing.hip", "quant.hip", "moe_gemm.hip", "fused_moe.hip"]
+SOURCES = ["fr_error.hip", "gating.hip", "routing.hip", "quant.hip", "moe_gemm.hip", "fused_moe.hip"] + [
+    "moe_gemm_inst_%s_%s.hip" % (t, e) for t in ("bf16", "f16", "fp8") for e in ("silu", "plain", "down")]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
@@ -49,7 +50,7 @@ def build(verbose: bool = False) -> str:
         src, obj = pair
         return _run([hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
 
-    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(os.cpu_count() or 8, 16, len(SOURCES))) as pool:
         for out in pool.map(one, zip(SOURCES, objs)):
             if verbose and out.strip():
                 print(out)

@@ -1,5 +1,5 @@
 // Host side of the grouped expert GEMMs: tile selection, launches, top-k combine.
-#include "moe_gemm_persistent.h"
+#include "moe_gemm_tiles.h"
 #include "moe_gemv.h"
 
 namespace fr {
@@ -30,101 +30,15 @@ __global__ __launch_bounds__(256) void combine_kernel(const P* __restrict__ part
   *reinterpret_cast<typename Elem<T>::out4*>(out + idx) = o;
 }
 
-// ---- host side ----------------------------------------------------------------
-// Token-block sizes and their tile shapes.  K tiles are 128 bytes per row (256 for
-// the 16-row block); every block except 64 streams tiles HBM -> LDS directly.
-//   256 / 128 rows: 8 wavefronts, 32x32 MFMA, 2- or 3-slot ring (compute-bound regime);
-//                   in the 256-row tile one wavefront per SIMD issues the loads of both;
-//   64 rows:        3-slot ring, 8 wavefronts (4 with 256-byte row segments for the gate/up GEMM);
-//                   (the register-staged double buffer of STAGES == 0 is no longer used by any tile);
-//   32 / 16 rows:   decode regime, 16x16 MFMA, 3-slot ring, two workgroups per CU:
-//                   weight streaming at HBM rate.  The gate/up GEMM (short weight rows
-//                   of H elements, many of them) streams faster with 512-byte row
-//                   segments: T32L / T16L, used when H allows.
-template <typename T> struct Tiles {  // bf16 / fp16
-  typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
-  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
-  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;  // persistent form; one wavefront per SIMD issues the loads (2-4 % over each its own)
-  typedef Cfg<64, 256, 128, 2, 4, 32, 1, 3, 3> T64;    // 3-slot ring like the 128-row tile (5 % over the register-staged form)
-  typedef Cfg<64, 128, 256, 2, 2, 32, 1, 3> T64U;      // gate/up: 256-byte row segments, 4 wavefronts (another 5 %)
-  typedef Cfg<32, 128, 128, 1, 4, 16, 2, 3> T32;
-  typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
-  typedef Cfg<32, 128, 512, 1, 4, 16, 1, 2> T32L;
-  typedef Cfg<16, 64, 512, 1, 2, 16, 2, 2> T16L;
-};
-template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per two K-steps
-  typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
-  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
-  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;
-  typedef Cfg<64, 256, 128, 2, 4, 32, 1, 3, 3> T64;
-  typedef Cfg<64, 128, 256, 2, 2, 32, 1, 3> T64U;
-  typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;
-  typedef Cfg<16, 64, 256, 1, 2, 16, 2, 3> T16;
-  typedef Cfg<32, 128, 512, 1, 4, 16, 1, 2> T32L;
-  typedef Cfg<16, 64, 512, 1, 2, 16, 2, 2> T16L;
-};
-
-bool valid_block(int block) { return block == 16 || block == 32 || block == 64 || block == 128 || block == 256; }
-int elem_bytes(int dtype) { return dtype == FR_FP8_E4M3 ? 1 : 2; }
-int tile_k_bytes(int block, int dtype) { return (block == 16 || (block == 32 && dtype == FR_FP8_E4M3)) ? 256 : 128; }
-int k_multiple(int dtype, int block) { return tile_k_bytes(block, dtype) / elem_bytes(dtype); }
-
-template <typename T, int EPI>
-int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStream_t st) {
-  typedef Tiles<T> TL;
-  auto fill = [&](int BT, int BF, int bkb) {
-    const int bk = bkb / static_cast<int>(sizeof(T));
-    a.num_t_blocks = static_cast<int>(ceil_div(sorted_len, BT));
-    const int fper = (EPI == EPI_SILU) ? BF / 2 : BF;
-    a.num_f_tiles = static_cast<int>(ceil_div(a.N, fper));
-    a.group_t = BT >= 64 ? 4 : 8;
-    a.k_per_split = static_cast<int>(round_up(ceil_div(a.K, splits), bk));
-  };
-  switch (block) {
-    case 256:
-      fill(256, TL::T256::BF, TL::T256::BKB);
-      // One workgroup per CU: the persistent form hides each tile's ring fill and drain behind its
-      // neighbour's.  fp8 runs it with one fragment buffer (registers for the second address set): 4-5 %
-      // faster for the down projection, but 6 % slower for the gate/up GEMM (short K, register-starved
-      // epilogue: the hand-off K tiles spill; without the hand-off it is within 1 % of the plain kernel),
-      // which keeps the plain kernel.
-      if constexpr (sizeof(T) == 1 && EPI == EPI_SILU) return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
-      else return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
-    case 128:
-      fill(128, TL::T128::BF, TL::T128::BKB);
-      // The gate/up GEMM always takes the persistent form (its walk by expert fetches each expert's
-      // weights once per chunk of token blocks); the down projection of the layer (few feature tiles,
-      // long K) takes it for the split of the last round, a plain grouped GEMM keeps the plain kernel.
-      if constexpr (EPI != EPI_SILU) {
-        if (a.long_k) return launch_gemm_persistent<T, typename TL::T128P, EPI>(a, splits, st);
-      } else {
-        return launch_gemm_persistent<T, typename TL::T128P, EPI>(a, splits, st);
-      }
-      return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
-    case 64:
-      if (EPI == EPI_SILU && a.K % (TL::T64U::BKB / static_cast<int>(sizeof(T))) == 0) {
-        fill(64, TL::T64U::BF, TL::T64U::BKB);
-        return launch_gemm<T, typename TL::T64U, EPI>(a, splits, st);
-      }
-      fill(64, TL::T64::BF, TL::T64::BKB);
-      return launch_gemm<T, typename TL::T64, EPI>(a, splits, st);
-    case 32:
-      if (EPI == EPI_SILU && a.K % (TL::T32L::BKB / static_cast<int>(sizeof(T))) == 0) {
-        fill(32, TL::T32L::BF, TL::T32L::BKB);
-        return launch_gemm<T, typename TL::T32L, EPI>(a, splits, st);
-      }
-      fill(32, TL::T32::BF, TL::T32::BKB);
-      return launch_gemm<T, typename TL::T32, EPI>(a, splits, st);
-    case 16:
-      if (EPI == EPI_SILU && a.K % (TL::T16L::BKB / static_cast<int>(sizeof(T))) == 0) {
-        fill(16, TL::T16L::BF, TL::T16L::BKB);
-        return launch_gemm<T, typename TL::T16L, EPI>(a, splits, st);
-      }
-      fill(16, TL::T16::BF, TL::T16::BKB);
-      return launch_gemm<T, typename TL::T16, EPI>(a, splits, st);
-    default: return fail(FR_E_SHAPE, "routing block %d not in {16, 32, 64, 128, 256}", block);
-  }
-}
+// ---- tile launches: instantiated per (element type, epilogue) in moe_gemm_inst_*.hip ---------
+#define FR_DECLARE_TILES(T)                                                                       \
+  extern template int dispatch_block<T, EPI_PLAIN>(GemmArgs, int, int, int64_t, hipStream_t);     \
+  extern template int dispatch_block<T, EPI_SILU>(GemmArgs, int, int, int64_t, hipStream_t);      \
+  extern template int dispatch_block<T, EPI_DOWN>(GemmArgs, int, int, int64_t, hipStream_t);
+FR_DECLARE_TILES(bf16_t)
+FR_DECLARE_TILES(f16_t)
+FR_DECLARE_TILES(fp8_t)
+#undef FR_DECLARE_TILES
 
 template <int EPI>
 int dispatch_dtype(const GemmArgs& a, int dtype, int block, int splits, int64_t sorted_len, hipStream_t st) {

@@ -1,0 +1,6 @@
+// Grouped expert GEMM tiles for bf16 operands, EPI_DOWN epilogue.
+#include "moe_gemm_tiles.h"
+
+namespace fr {
+template int dispatch_block<bf16_t, EPI_DOWN>(GemmArgs, int, int, int64_t, hipStream_t);
+}  // namespace fr

@@ -149,3 +149,26 @@ def test_route_gate_large_batch(native, E, topk, H):
     assert flips.float().mean() < 0.02
     ok = ~flips.any(dim=1)
     torch.testing.assert_close(w.cpu()[ok], ow[ok], atol=1e-4, rtol=0)
+
+
+@pytest.mark.parametrize("E,topk,H", [(16, 2, 4096), (128, 4, 1024), (100, 3, 512)])
+def test_fused_route_half_and_int64_buffers(native, E, topk, H):
+    """The reference's own recipe hands fused_route fp16 weight and int64 id buffers of [M, E]
+    (tests/test_route.py:30-38) and allows up to 128 experts (ops/stable_route.py:130-134):
+    both must give the fp32-logit result, not one rounded to the operand type first."""
+    from fast_route_amd.ops.stable_route import fused_route
+    for M in (3, 257):
+        _say(f"fused_route fp16/int64 buffers E={E} k={topk} H={H} M={M}")
+        g = torch.Generator().manual_seed(E * 31 + H + M)
+        h = (torch.randn(M, H, generator=g) / 10).half()
+        gate = (torch.randn(H, E, generator=g) / 10).half()
+        tw = torch.empty(M, E, dtype=torch.float16, device="cuda")
+        ti = torch.empty(M, E, dtype=torch.int64, device="cuda")
+        w, ids = fused_route(h.cuda(), gate.cuda(), topk, tw, ti, True)
+        torch.cuda.synchronize()
+        assert w.dtype == torch.float16 and ids.dtype == torch.int64 and w.shape == ids.shape == (M, topk)
+        ow, oid = oracle.gating_topk((h.double() @ gate.double()).float(), topk, True)
+        flips = (ids.cpu() != oid.long())
+        assert flips.float().mean() < 0.02   # fp32 against float64 logits: near-ties only
+        ok = ~flips.any(dim=1)
+        torch.testing.assert_close(w.cpu().float()[ok], ow[ok], atol=1e-3, rtol=0)  # fp16 storage of the weights
