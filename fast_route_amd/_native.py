@@ -43,6 +43,8 @@ SIGNATURES = {
                                         c_void_p, c_void_p, c_void_p]),
     "fr_fused_moe_fp8": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64,
                                  c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_void_p]),
+    "fr_fused_moe_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int,
+                                     c_int, c_int, c_void_p, c_void_p]),
     "fr_fused_moe": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int,
                              c_int, c_int, c_void_p, c_void_p, c_int64, c_void_p]),
 }

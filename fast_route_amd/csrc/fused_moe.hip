@@ -217,3 +217,50 @@ extern "C" int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, con
   return fr_moe_down_combine_fp8(c.actq, c.act_scale, w2q, w2_scale, c.topk_w, c.sorted, c.expert_ids, c.npost, M, H, F, E,
                                  topk, p.block, p.split_k, x_dtype, c.partial, out, c.tail, stream);
 }
+
+// ---- one entry point that allocates nothing ------------------------------------
+// The layer's scratch lives in a device array of this library instead of a caller's buffer.
+// Host code may not pass the array's name to a kernel (on the host it is a stand-in, not a
+// device address): its address on the current device is looked up once per device and kept.
+namespace fr {
+namespace {
+constexpr int64_t kStaticScratchBytes = int64_t(64) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+int static_scratch(void** out) {
+  constexpr int kMaxDevices = 64;
+  static void* ptrs[kMaxDevices] = {};  // per device; two threads racing here store the same address
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(FR_E_NO_DEVICE, "fr_fused_moe_noalloc: device %d (%s)", dev, hipGetErrorString(e));
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return fail(FR_E_NO_DEVICE, "fr_fused_moe_noalloc: hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    }
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return FR_OK;
+}
+}  // namespace
+}  // namespace fr
+
+extern "C" int fr_fused_moe_noalloc(const void* x, const void* w1, const void* w2, const void* logits, int logits_dtype,
+                                    int64_t M, int64_t H, int64_t F, int E, int topk, int renormalize, int dtype,
+                                    void* out, void* stream) {
+  fr_moe_plan p;
+  int rc = fr_moe_get_plan(M, H, F, E, topk, dtype, &p);
+  if (rc != FR_OK) return rc;
+  FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "fr_fused_moe_noalloc: dtype %d not in {f16, bf16}", dtype);
+  FR_REQUIRE(p.workspace_bytes <= kStaticScratchBytes, FR_E_WORKSPACE,
+             "fr_fused_moe_noalloc: these sizes need %lld bytes of scratch, the library's static scratch holds %lld; use fr_fused_moe with a workspace",
+             (long long)p.workspace_bytes, (long long)kStaticScratchBytes);
+  if (M == 0) return FR_OK;
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc != FR_OK) return rc;
+  return fr_fused_moe(x, w1, w2, logits, logits_dtype, M, H, F, E, topk, renormalize, dtype, out, ws, kStaticScratchBytes, stream);
+}

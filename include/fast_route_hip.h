@@ -155,6 +155,20 @@ int fr_fused_moe(const void* x, const void* w1, const void* w2, const void* logi
                  int renormalize, int dtype, void* out, void* workspace, int64_t workspace_bytes,
                  void* stream);
 
+/* fr_fused_moe without a workspace argument and without any allocation: the layer's
+ * scratch (top-k arrays, routing arrays, activated intermediate, partial rows) lives in a
+ * 64 MiB device array inside this library, which every GPU the library runs on holds
+ * until the process ends.  No counterpart in the reference; it is for callers that
+ * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  Sizes whose fr_moe_get_plan().workspace_bytes exceed 64 MiB are
+ * rejected with FR_E_WORKSPACE (Mixtral-8x7B shape: up to 207 tokens).  The array's
+ * device address is looked up on the first call on each device (with that device
+ * current); nothing in the array has to start at zero.  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (two streams, two threads) race. */
+int fr_fused_moe_noalloc(const void* x, const void* w1, const void* w2, const void* logits,
+                         int logits_dtype, int64_t M, int64_t H, int64_t F, int E, int topk,
+                         int renormalize, int dtype, void* out, void* stream);
+
 /* ---- fp8 (OCP e4m3fn) path -------------------------------------------------
  * No counterpart in the reference (its only fp8 mentions are commented autotune
  * rows, fast_route/fast_route/ops/stable_route.py:20-28); defined by the fp8
