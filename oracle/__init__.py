@@ -17,6 +17,7 @@ from .moe_oracle import (  # noqa: F401
     e4m3fn_decode_table,
     e4m3fn_encode,
     quant_e4m3_rows,
+    quantize_weights_fp8,
     fused_moe_fp8,
     make_inputs,
     zipf_logits,

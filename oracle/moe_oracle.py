@@ -31,6 +31,8 @@ from __future__ import annotations
 
 import math
 
+import os
+
 import numpy as np
 import torch
 import torch.nn.functional as F
@@ -206,27 +208,40 @@ def e4m3fn_decode_table() -> np.ndarray:
     return out
 
 
-def e4m3fn_encode(x: np.ndarray) -> np.ndarray:
-    """Round-to-nearest-even fp32 -> e4m3fn code (uint8), saturating at +-448."""
-    x = np.asarray(x, dtype=np.float32)
+def _e4m3fn_encode_block(x: np.ndarray) -> np.ndarray:
     sign = (np.signbit(x)).astype(np.uint8) << 7
-    a = np.minimum(np.abs(x).astype(np.float64), 448.0)
+    a = np.minimum(np.abs(x), np.float32(448.0))  # float32 throughout: every scaling below is by a power of two, hence exact
     # exponent of the quantisation step: normal numbers have 3 mantissa bits,
-    # everything below 2**-6 shares the subnormal step 2**-9.
-    with np.errstate(divide="ignore"):
-        ex = np.floor(np.log2(np.where(a > 0, a, 1.0)))
-    ex = np.maximum(ex, -6.0)
-    step = 2.0 ** (ex - 3)
-    q = np.rint(a / step)  # numpy rint is round-half-even
-    val = q * step  # may carry into the next binade; re-derive fields from val
-    with np.errstate(divide="ignore"):
-        ev = np.floor(np.log2(np.where(val > 0, val, 1.0)))
-    ev = np.maximum(ev, -6.0)
-    is_sub = val < 2.0 ** -6
-    mant = np.where(is_sub, val / 2.0 ** -9, (val / 2.0 ** ev - 1.0) * 8.0)
-    expo = np.where(is_sub, 0.0, ev + 7.0)
-    code = (expo.astype(np.int64) << 3) | np.rint(mant).astype(np.int64)
+    # everything below 2**-6 shares the subnormal step 2**-9.  frexp: a = m * 2**e, m in [0.5, 1).
+    _, e = np.frexp(a)
+    ex = np.maximum(e - 1, -6)
+    q = np.rint(np.ldexp(a, 3 - ex))  # numpy rint is round-half-even
+    val = np.ldexp(q, ex - 3)  # may carry into the next binade; re-derive fields from val
+    _, e2 = np.frexp(val)
+    ev = np.maximum(e2 - 1, -6)
+    is_sub = val < np.float32(2.0 ** -6)
+    mant = np.where(is_sub, np.ldexp(val, 9), (np.ldexp(val, -ev) - np.float32(1.0)) * np.float32(8.0))
+    expo = np.where(is_sub, 0, ev + 7)
+    code = (expo.astype(np.int32) << 3) | np.rint(mant).astype(np.int32)
     return (code.astype(np.uint8) | sign).astype(np.uint8)
+
+
+def e4m3fn_encode(x: np.ndarray) -> np.ndarray:
+    """Round-to-nearest-even fp32 -> e4m3fn code (uint8), saturating at +-448.
+    Large inputs go through in blocks of rows to bound the temporaries."""
+    x = np.asarray(x, dtype=np.float32)
+    if x.ndim < 2 or x.size <= (1 << 24):
+        return _e4m3fn_encode_block(x)
+    out = np.empty(x.shape, dtype=np.uint8)
+    rows = max(1, (1 << 22) // max(1, x[0].size))
+
+    def one(r0):
+        out[r0:r0 + rows] = _e4m3fn_encode_block(x[r0:r0 + rows])
+
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=min(16, os.cpu_count() or 1)) as pool:  # numpy releases the GIL inside its loops
+        list(pool.map(one, range(0, x.shape[0], rows)))
+    return out
 
 
 def quant_e4m3_rows(x: torch.Tensor):
@@ -239,19 +254,30 @@ def quant_e4m3_rows(x: torch.Tensor):
     return codes, scale
 
 
-def fused_moe_fp8(hidden_states, w1, w2, gating_output, topk: int, renormalize: bool = True):
+def quantize_weights_fp8(w1, w2):
+    """(w1 codes, w1 scales, w2 codes, w2 scales) per (expert, output channel): what the fp8 layer's
+    weight preparation produces; fused_moe_fp8 takes it as `weights_q` to quantise large weights once."""
+    E, F2, H = w1.shape
+    w1c, w1s = quant_e4m3_rows(w1.reshape(E * F2, H))
+    w2c, w2s = quant_e4m3_rows(w2.reshape(E * w2.shape[1], w2.shape[2]))
+    return w1c, w1s, w2c, w2s
+
+
+def fused_moe_fp8(hidden_states, w1, w2, gating_output, topk: int, renormalize: bool = True, weights_q=None):
     """fp8 layer as the fp8 Mixtral workload defines it: weights quantised per (expert,
     output channel), activations per token (both before the gate/up GEMM and
     before the down GEMM), everything dequantised to fp32 and run through the
     fp32 oracle.  Returns (out fp32, dict with the quantised operands)."""
-    table = torch.from_numpy(e4m3fn_decode_table())
     E, F2, H = w1.shape
-    w1c, w1s = quant_e4m3_rows(w1.reshape(E * F2, H))
-    w2c, w2s = quant_e4m3_rows(w2.reshape(E * w2.shape[1], w2.shape[2]))
-    w1d = (table[torch.from_numpy(w1c).long()] * torch.from_numpy(w1s)[:, None]).reshape(E, F2, H)
-    w2d = (table[torch.from_numpy(w2c).long()] * torch.from_numpy(w2s)[:, None]).reshape(w2.shape)
+    w1c, w1s, w2c, w2s = weights_q if weights_q is not None else quantize_weights_fp8(w1, w2)
+    tab = e4m3fn_decode_table()
+    Hd = w2.shape[1]
+
+    def dequant(codes, scales):  # uint8 codes index the 256-entry table directly
+        return torch.from_numpy(tab[codes] * scales[:, None])
+
     xc, xs = quant_e4m3_rows(hidden_states)
-    xd = table[torch.from_numpy(xc).long()] * torch.from_numpy(xs)[:, None]
+    xd = dequant(xc, xs)
     wts, ids = gating_topk(gating_output, topk, renormalize)
     M, k = ids.shape
     out = torch.zeros(M, H, dtype=torch.float32)
@@ -260,10 +286,13 @@ def fused_moe_fp8(hidden_states, w1, w2, gating_output, topk: int, renormalize: 
         tok, slot = (idl == e).nonzero(as_tuple=True)
         if tok.numel() == 0:
             continue
-        a = silu_and_mul(xd[tok] @ w1d[e].T).to(torch.bfloat16)  # kernel stores bf16 then requantises
+        w1d = dequant(w1c[e * F2:(e + 1) * F2], w1s[e * F2:(e + 1) * F2])  # one expert at a time bounds the memory
+        a = silu_and_mul(xd[tok] @ w1d.T).to(torch.bfloat16)  # kernel stores bf16 then requantises
+        del w1d
         ac, asc = quant_e4m3_rows(a)
-        ad = table[torch.from_numpy(ac).long()] * torch.from_numpy(asc)[:, None]
-        out.index_add_(0, tok, (ad @ w2d[e].T) * wts[tok, slot].unsqueeze(1))
+        ad = dequant(ac, asc)
+        w2d = dequant(w2c[e * Hd:(e + 1) * Hd], w2s[e * Hd:(e + 1) * Hd])
+        out.index_add_(0, tok, (ad @ w2d.T) * wts[tok, slot].unsqueeze(1))
     return out, {"w1_codes": w1c.reshape(E, F2, H), "w1_scale": w1s.reshape(E, F2),
                  "w2_codes": w2c.reshape(w2.shape), "w2_scale": w2s.reshape(E, -1),
                  "x_codes": xc, "x_scale": xs}

@@ -97,6 +97,7 @@ def test_fp8_mixtral_shape_sampled(native):
     w2 = (torch.randn(E, H, Fd, generator=g, device="cuda") * 0.02).bfloat16()
     w1q, w1s, w2q, w2s = prepare_weights_fp8(w1, w2)
     w1c, w2c = w1.cpu(), w2.cpu()
+    wq = oracle.quantize_weights_fp8(w1c, w2c)  # once: 1.4e9 weights through the CPU encoder
     for M in (16, 128, 256, 4096):
         _say(f"fp8 mixtral M={M}")
         x = torch.randn(M, H, generator=g, device="cuda").bfloat16()
@@ -104,7 +105,7 @@ def test_fp8_mixtral_shape_sampled(native):
         out = fused_moe_fp8(x, w1q, w1s, w2q, w2s, logits, k, True)
         torch.cuda.synchronize()
         sample = torch.arange(0, M, max(1, M // 12))[:12]
-        ref, _ = oracle.fused_moe_fp8(x[sample].cpu(), w1c, w2c, logits[sample].cpu(), k, True)
+        ref, _ = oracle.fused_moe_fp8(x[sample].cpu(), w1c, w2c, logits[sample].cpu(), k, True, weights_q=wq)
         o = out[sample].float().cpu()
         assert (o - ref).norm() / ref.norm() <= 1e-2
         out2 = fused_moe_fp8(x, w1q, w1s, w2q, w2s, logits, k, True)

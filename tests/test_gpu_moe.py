@@ -65,13 +65,23 @@ def test_fine_grained_config(native, M):
 
 
 def test_fine_grained_full_width(native):
-    """Config 4's real H2048 / F1408 at M=128."""
+    """The fine-grained workload at its real H2048 / F1408 / E64 / top-6 with Zipf-skewed load, every token
+    count of its sweep: all tokens against the oracle up to 512, a sample of 48 tokens above."""
     from fast_route_amd import fused_moe
-    _say("layer C4 full width M=128")
-    x, logits, w1, w2 = _inputs(128, 2048, 1408, 64, 5, torch.bfloat16, zipf=True)
-    out = fused_moe(x.cuda(), w1.cuda(), w2.cuda(), logits.cuda(), 6, True)
-    torch.cuda.synchronize()
-    _assert_close(out, oracle.fused_moe(x, w1, w2, logits, 6, True), torch.bfloat16, "C4 full")
+    H, Fd, E, k = 2048, 1408, 64, 6
+    _, _, w1, w2 = _inputs(1, H, Fd, E, 5, torch.bfloat16)
+    w1d, w2d = w1.cuda(), w2.cuda()
+    for M in (1, 32, 128, 512, 2048, 8192):
+        _say(f"layer C4 full width M={M}")
+        g = torch.Generator().manual_seed(500 + M)
+        x = torch.randn(M, H, generator=g).bfloat16()
+        logits = oracle.zipf_logits(M, E, 600 + M)
+        out = fused_moe(x.cuda(), w1d, w2d, logits.cuda(), k, True)
+        torch.cuda.synchronize()
+        assert torch.isfinite(out.float()).all()
+        sample = torch.arange(M) if M <= 512 else torch.arange(0, M, M // 48)[:48]
+        ref = oracle.fused_moe(x[sample], w1, w2, logits[sample], k, True)
+        _assert_close(out[sample], ref, torch.bfloat16, f"C4 full M={M}")
 
 
 def test_layer_edge_cases(native):
@@ -438,6 +448,16 @@ def test_profile_twin_matches_layer_and_writes_trace(native, tmp_path):
     out = profile_fused_route.fused_moe(x.cuda(), gate.cuda(), w1.cuda(), w2.cuda(), k, True, save_dir=str(tmp_path))
     torch.cuda.synchronize()
     assert torch.equal(out, ref)
+    # and against the oracle: routing from fp64 logits; tokens whose fp32 near-tie flipped an id are left out
+    ow, oid = oracle.route_from_gate(x, gate, k)
+    from fast_route_amd.ops.stable_route import fused_route
+    tw = torch.empty(M, k, dtype=torch.float32, device="cuda")
+    ti = torch.empty(M, k, dtype=torch.int32, device="cuda")
+    _, ids = fused_route(x.cuda(), gate.cuda(), k, tw, ti, True)
+    same = (ids.cpu() == oid).all(dim=1)
+    assert same.float().mean() > 0.95
+    want = oracle.moe_experts(x, w1, w2, ow, oid)
+    _assert_close(out[same.cuda()], want[same], dtype, "profile twin vs oracle")
     path = tmp_path / f"fused_breakdown_{M}_{H}_{E}_{2 * Fd}_{k}.json"
     trace = json.loads(path.read_text())
     names = [e["name"] for e in trace["traceEvents"]]
@@ -463,11 +483,23 @@ def test_transformer_layer_bench_runs_and_matches_its_parts(native):
         h = (attn(x) + x).view(-1, 512)
         again = fused_moe(h, gate, w1, w2, 2, True, False)
     assert torch.equal(out, again)
+    # against the oracle: the MoE of the layer's own attention output, routed and multiplied on the CPU
+    hc, gc = h.cpu(), gate.cpu()
+    ow, oid = oracle.route_from_gate(hc, gc, 2)
+    from fast_route_amd.ops.stable_route import fused_route
+    tw = torch.empty(h.shape[0], 2, dtype=torch.float32, device="cuda")
+    ti = torch.empty(h.shape[0], 2, dtype=torch.int32, device="cuda")
+    _, ids = fused_route(h, gate, 2, tw, ti, True)
+    same = (ids.cpu() == oid).all(dim=1)
+    assert same.float().mean() > 0.95
+    want = oracle.moe_experts(hc, w1.cpu(), w2.cpu(), ow, oid)
+    _assert_close(out[same.cuda()], want[same], torch.float16, "transformer layer vs oracle")
 
 
 def test_mixtral_shape_sampled_tokens_and_properties(native):
-    """Mixtral-8x7B shape at full size (H4096 F14336 E8 top2): oracle on a sample of
-    tokens, plus size-independent properties on all of them."""
+    """Mixtral-8x7B shape at full size (H4096 F14336 E8 top2), every token count of its sweep:
+    oracle on a sample of tokens and determinism; at 16 and 4096 tokens also the size-independent
+    properties (batch independence, linearity in the routed weights) on all tokens."""
     from fast_route_amd import fused_moe, fused_experts
     dtype = torch.bfloat16
     H, Fd, E, k = 4096, 14336, 8, 2
@@ -475,7 +507,7 @@ def test_mixtral_shape_sampled_tokens_and_properties(native):
     w1 = (torch.randn(E, 2 * Fd, H, generator=g, device="cuda") * 0.02).to(dtype)
     w2 = (torch.randn(E, H, Fd, generator=g, device="cuda") * 0.02).to(dtype)
     w1c, w2c = w1.cpu(), w2.cpu()
-    for M in (16, 4096):
+    for M in (1, 16, 64, 256, 1024, 4096, 16384):
         _say(f"mixtral full width M={M}")
         x = torch.randn(M, H, generator=g, device="cuda").to(dtype)
         logits = torch.randn(M, E, generator=g, device="cuda")
@@ -488,6 +520,8 @@ def test_mixtral_shape_sampled_tokens_and_properties(native):
         # determinism: same call, same bits
         out2 = fused_moe(x, w1, w2, logits, k, True)
         assert torch.equal(out, out2)
+        if M not in (16, 4096):
+            continue
         # a token's output does not depend on which other tokens share the batch
         half = fused_moe(x[: M // 2].contiguous(), w1, w2, logits[: M // 2].contiguous(), k, True)
         _assert_close(half, out[: M // 2].float().cpu(), dtype, "batch independence")
@@ -499,6 +533,27 @@ def test_mixtral_shape_sampled_tokens_and_properties(native):
         a = fused_experts(x, w1, w2, w, ids)
         b = fused_experts(x, w1, w2, 2 * w, ids)
         assert torch.equal(a, out) and torch.equal(b.float(), 2 * a.float())
+
+
+@pytest.mark.parametrize("m", [1, 33, 222, 1024])
+def test_reference_end_to_end_recipe(native, m):
+    """The reference's own end-to-end check replayed (benchmarks/swizzle_moe/perf_test_moe.py:34-73):
+    fp16 operands drawn as randn / 10, routing = torch.topk(softmax(randn score)), no renormalisation,
+    experts-only entry point, torch_moe as the expectation, assert_close(atol=1e-2, rtol=0).
+    Widths are scaled down from the reference's n=14336 / k=4096 to keep the CPU expectation quick."""
+    from fast_route_amd import fused_experts
+    n, k, e, topk = 1024, 512, 8, 2
+    _say(f"reference recipe m={m} n={n} k={k} e={e} topk={topk}")
+    torch.manual_seed(3227)  # the reference's seed for this check
+    a = (torch.randn((m, k)) / 10).half()
+    w1 = (torch.randn((e, 2 * n, k)) / 10).half()
+    w2 = (torch.randn((e, k, n)) / 10).half()
+    score = torch.softmax(torch.randn((m, e)), dim=-1)
+    topk_weight, topk_ids = torch.topk(score, topk)
+    out = fused_experts(a.cuda(), w1.cuda(), w2.cuda(), topk_weight.cuda(), topk_ids.cuda(), inplace=False)
+    torch.cuda.synchronize()
+    want = oracle.moe_experts(a, w1, w2, topk_weight, topk_ids)
+    torch.testing.assert_close(out.float().cpu(), want, atol=1e-2, rtol=0)
 
 
 def test_random_shapes_against_oracle(native):

@@ -315,3 +315,50 @@ def test_reciprocal_fma_quotient_is_correctly_rounded():
             assert got.view(np.uint32) == rn32(F(float(x)) / F(float(s))).view(np.uint32), (kind, x, a)
             checked += 1
     assert checked > 8000
+
+
+def test_fp8_layer_oracle_against_independent_per_pair_loop():
+    """oracle.fused_moe_fp8 restated pair by pair on torch.float8_e4m3fn casts and torch.topk:
+    scale per ROW (weight output channel, token, activated row), bf16 rounding of the activated
+    row before it is quantised again, routed weight after the down projection.  A per-tensor scale,
+    a skipped bf16 rounding or a skipped re-quantisation each move the result by far more than the
+    fp32 summation-order difference allowed here."""
+    def q(t):  # per-row e4m3 quantise + dequantise with fp32 scale amax/448
+        amax = t.abs().amax(dim=-1, keepdim=True)
+        s = torch.where(amax > 0, amax / 448.0, torch.ones_like(amax))
+        return (t / s).to(torch.float8_e4m3fn).float() * s
+
+    def layer(x, logits, w1, w2, k, mistake=None):
+        M, H = x.shape
+        E, F2, _ = w1.shape
+        Fd = F2 // 2
+        if mistake == "per_tensor_scale":
+            s1, s2 = w1.abs().max() / 448.0, w2.abs().max() / 448.0
+            w1q, w2q = (w1 / s1).to(torch.float8_e4m3fn).float() * s1, (w2 / s2).to(torch.float8_e4m3fn).float() * s2
+        else:
+            w1q, w2q = q(w1.reshape(E * F2, H)).reshape(E, F2, H), q(w2.reshape(E * H, Fd)).reshape(E, H, Fd)
+        xq = q(x)
+        pw, pid = torch.topk(torch.softmax(logits.float(), -1), k)  # no ties in these random logits
+        pw = pw / pw.sum(-1, keepdim=True)
+        want = torch.zeros(M, H)
+        for m in range(M):
+            for j in range(k):
+                e = int(pid[m, j])
+                h = w1q[e] @ xq[m]
+                a = torch.nn.functional.silu(h[:Fd]) * h[Fd:]
+                if mistake != "no_bf16_rounding":
+                    a = a.bfloat16().float()
+                if mistake != "no_requantisation":
+                    a = q(a[None, :])[0]
+                want[m] += float(pw[m, j]) * (w2q[e] @ a)
+        return want
+
+    for seed, (M, H, Fd, E, k) in enumerate([(7, 32, 16, 4, 2), (5, 64, 32, 3, 3), (9, 16, 48, 8, 1)]):
+        x, logits, w1, w2 = oracle.make_inputs(M, H, Fd, E, seed=40 + seed, w_std=0.1)
+        x, w1, w2 = x.bfloat16().float(), w1.bfloat16().float(), w2.bfloat16().float()
+        got, _ = oracle.fused_moe_fp8(x, w1, w2, logits, k, True)
+        want = layer(x, logits, w1, w2, k)
+        tol = 1e-5 * want.abs().max()
+        assert (got - want).abs().max() <= tol, (got - want).abs().max()
+        for mistake in ("per_tensor_scale", "no_bf16_rounding", "no_requantisation"):
+            assert (got - layer(x, logits, w1, w2, k, mistake)).abs().max() > 20 * tol, mistake
