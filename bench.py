@@ -1,6 +1,7 @@
 """Benchmark of the fused MoE layer on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens M] [--no-sweep] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens M] [--no-sweep] [--no-cpu] [--no-configs]
+    python bench.py -n 8192 -k 4096 -e 16 --topk 2 --reference-protocol      (the reference's own sweep, fp16 randn/10)
 
 A step is one pass of the whole layer (gating -> routing arrays -> gate/up GEMM
 with SiLU*mul -> down GEMM with routed weight -> top-k combine) over one batch
@@ -9,10 +10,15 @@ Inputs and weights are resident in HBM before the timed region.  Prints ONE JSON
 line: the headline token count (default 4096), the per-stage times measured with
 events on the launch stream, the roofline of the dominant kernel, the token sweep
 and the CPU baseline (the fp32 PyTorch oracle on the host cores, bounded sample).
+Unless --no-configs is given the same line also carries compact records of the other
+workloads: the small layer (caches flushed between repetitions), the routing-only stress
+case (bit-exact flag), the fine-grained many-expert sweep and the fp8 sweep, each with
+its bound, roofline fraction and the error of one point against the CPU oracle.
 """
 from __future__ import annotations
 
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -47,13 +53,15 @@ def layer_bytes(M, H, F, E, topk, active, bw=2, ba=2):
 class Layer:
     """Device buffers + staged calls through the C ABI for one (shape, M)."""
 
-    def __init__(self, torch, N, shape, M, w1, w2, seed, fp8=None):
+    def __init__(self, torch, N, shape, M, w1, w2, seed, fp8=None, dtype=None, x_scale=1.0):
         self.torch, self.N, self.M = torch, N, M
+        self.tdtype = dtype or torch.bfloat16
+        self.code = N.dtype_code(self.tdtype)
         self.fp8 = fp8  # (w1q, w1_scale, w2q, w2_scale) or None
         self.H, self.F, self.E, self.topk = shape["H"], shape["F"], shape["E"], shape["topk"]
         dev = "cuda"
         g = torch.Generator(device=dev).manual_seed(seed + M)
-        self.x = torch.randn(M, self.H, generator=g, device=dev).to(torch.bfloat16)
+        self.x = (torch.randn(M, self.H, generator=g, device=dev) * x_scale).to(self.tdtype)
         if shape["zipf"]:
             r = (torch.randperm(self.E, generator=g, device=dev) + 1).double()
             pz = r.pow(-1.2)
@@ -62,10 +70,10 @@ class Layer:
             self.logits = torch.randn(M, self.E, generator=g, device=dev)
         self.w1, self.w2 = w1, w2
         self.plan = N.FrMoePlan()
-        N.check(N.lib().fr_moe_get_plan(M, self.H, self.F, self.E, self.topk, N.FR_FP8_E4M3 if fp8 else N.FR_BF16, self.plan))
+        N.check(N.lib().fr_moe_get_plan(M, self.H, self.F, self.E, self.topk, N.FR_FP8_E4M3 if fp8 else self.code, self.plan))
         p, n = self.plan, M * self.topk
         self.ws = torch.empty(max(p.workspace_bytes, 256), dtype=torch.uint8, device=dev)
-        self.out = torch.empty(M, self.H, dtype=torch.bfloat16, device=dev)
+        self.out = torch.empty(M, self.H, dtype=self.tdtype, device=dev)
         # staged buffers
         self.tw = torch.empty(n, dtype=torch.float32, device=dev)
         self.ti = torch.empty(n, dtype=torch.int32, device=dev)
@@ -74,7 +82,7 @@ class Layer:
         self.npost = torch.empty(1, dtype=torch.int32, device=dev)
         self.aws_bytes = N.lib().fr_moe_align_workspace_bytes(n, self.E)
         self.aws = torch.empty(max(self.aws_bytes, 256), dtype=torch.uint8, device=dev)
-        self.act = torch.empty(p.sorted_len, self.F, dtype=torch.bfloat16, device=dev)
+        self.act = torch.empty(p.sorted_len, self.F, dtype=self.tdtype, device=dev)
         self.partial = torch.empty(p.split_k * n * self.H, dtype=torch.float32, device=dev)
         self.tail = torch.empty(p.tail_bytes, dtype=torch.uint8, device=dev) if p.tail_bytes else None
         if fp8:
@@ -93,7 +101,7 @@ class Layer:
                                              self.topk, 1, self.out.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream))
             return
         N.check(N.lib().fr_fused_moe(self.x.data_ptr(), self.w1.data_ptr(), self.w2.data_ptr(), self.logits.data_ptr(),
-                                     N.FR_F32, self.M, self.H, self.F, self.E, self.topk, 1, N.FR_BF16,
+                                     N.FR_F32, self.M, self.H, self.F, self.E, self.topk, 1, self.code,
                                      self.out.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream))
 
     def staged(self, events=None):
@@ -124,13 +132,13 @@ class Layer:
             rec(4)
             return
         N.check(lib.fr_moe_gateup_silu(self.x.data_ptr(), self.w1.data_ptr(), self.sorted.data_ptr(), self.eids.data_ptr(),
-                                       self.npost.data_ptr(), self.M, self.H, self.F, self.E, self.topk, p.block, N.FR_BF16,
+                                       self.npost.data_ptr(), self.M, self.H, self.F, self.E, self.topk, p.block, self.code,
                                        self.act.data_ptr(), self.tail.data_ptr() if self.tail is not None else None,
                                        self.stream))
         rec(3)
         N.check(lib.fr_moe_down_combine(self.act.data_ptr(), self.w2.data_ptr(), self.tw.data_ptr(), self.sorted.data_ptr(),
                                         self.eids.data_ptr(), self.npost.data_ptr(), self.M, self.H, self.F, self.E,
-                                        self.topk, p.block, p.split_k, N.FR_BF16, self.partial.data_ptr(),
+                                        self.topk, p.block, p.split_k, self.code, self.partial.data_ptr(),
                                         self.out.data_ptr(), self.tail.data_ptr() if self.tail is not None else None,
                                         self.stream))
         rec(4)
@@ -139,29 +147,50 @@ class Layer:
         return int(self.torch.unique(self.ti).numel())
 
 
-def time_layer(torch, layer, steps, warmup):
+_FLUSH = {}
+
+
+def flush_caches(torch):
+    """Writes 512 MiB: twice the 256 MB Infinity Cache, so nothing of the layer's operands survives in it or in L2."""
+    if "buf" not in _FLUSH:
+        _FLUSH["buf"] = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
+    _FLUSH["buf"].fill_(1)
+
+
+def time_layer(torch, layer, steps, warmup, flush=False):
+    """flush: the weights fit the Infinity Cache (small workloads); every repetition then starts from cold caches
+    (one event pair per repetition, the flush outside it) instead of running back to back."""
     for _ in range(warmup):
         layer.fused()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        layer.fused()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    if flush:
+        wall_ms = None
+    else:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            layer.fused()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     # per-step spread (median, 20th and 80th percentile) from one event pair per step
     pe = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for a, b in pe:
+        if flush:
+            flush_caches(torch)
         a.record()
         layer.fused()
         b.record()
     torch.cuda.synchronize()
     per = sorted(a.elapsed_time(b) * 1e3 for a, b in pe)
     quant = {"p20": per[len(per) // 5], "p50": per[len(per) // 2], "p80": per[(4 * len(per)) // 5]}
+    if flush:
+        wall_ms = quant["p50"] / 1e3
     # per-stage times: the same kernels launched stage by stage with events on the launch stream
     evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(steps)]
     layer.staged()
     torch.cuda.synchronize()
     for s in range(steps):
+        if flush:
+            flush_caches(torch)
         layer.staged(evs[s])
     torch.cuda.synchronize()
     names = ["route", "moe_align", "moe_1+silu_and_mul", "moe_2+sum"]
@@ -170,11 +199,11 @@ def time_layer(torch, layer, steps, warmup):
     return wall_ms, stage_us, quant
 
 
-def measure(torch, N, shape, M, w1, w2, steps, warmup, seed, fp8=None):
-    layer = Layer(torch, N, shape, M, w1, w2, seed, fp8)
+def measure(torch, N, shape, M, w1, w2, steps, warmup, seed, fp8=None, flush=False, dtype=None, x_scale=1.0):
+    layer = Layer(torch, N, shape, M, w1, w2, seed, fp8, dtype=dtype, x_scale=x_scale)
     if fp8:  # pad rows of act beyond npost are never written: keep them finite for the staged quantisation
         layer.act.zero_()
-    wall_ms, stage_us, quant = time_layer(torch, layer, steps, warmup)
+    wall_ms, stage_us, quant = time_layer(torch, layer, steps, warmup, flush)
     H, F, E, topk = shape["H"], shape["F"], shape["E"], shape["topk"]
     active = layer.active_experts()
     fl = layer_flops(M, H, F, topk)
@@ -191,6 +220,8 @@ def measure(torch, N, shape, M, w1, w2, steps, warmup, seed, fp8=None):
         "stage_us": {k: round(v, 2) for k, v in stage_us.items()},
         "ref_2mnk_tflops": round(2.0 * M * F * H / t / 1e12, 3),
     }
+    if flush:
+        rec["cache_flush"] = "512 MiB written before every timed repetition"
     return rec, layer
 
 
@@ -223,22 +254,58 @@ def kernel_roofline(shape, rec, fp8=False):
             "avg_launch_us": round(dur * 1e6, 2), "algorithmic_bytes_per_launch": byts}
 
 
+def kernel_sources_sha():
+    """Hash of the HIP sources the library is built from: ties an offline counter record to the kernels it measured."""
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fast_route_amd", "csrc")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(root)):
+        if name.endswith((".h", ".hip")):
+            with open(os.path.join(root, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
 def recorded_traffic(metric):
     """HBM bytes per launch of the dominant kernel for this workload, as measured offline with
     rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE runs, scaled by the copy probe) and recorded
-    in profiles/hbm_traffic.json; None when the workload has no record."""
+    in profiles/hbm_traffic.json; None when the workload has no record or the record was taken
+    with other kernel sources than the ones present."""
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
     try:
         with open(path) as f:
-            rec = json.load(f).get(metric)
+            doc = json.load(f)
     except (OSError, ValueError):
         return None
-    return rec["traffic_bytes"] if rec else None
+    rec = doc.get(metric)
+    if not rec or doc.get("kernel_sources_sha") != kernel_sources_sha():
+        return None
+    return rec["traffic_bytes"]
+
+
+def host_cpu():
+    """(threads the CPU legs use, CPU model): the box's CPU share when the environment states one, else every core."""
+    n = os.cpu_count() or 1
+    try:
+        n = min(n, int(os.environ.get("OMP_NUM_THREADS", n)))
+    except ValueError:
+        pass
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return max(n, 1), model
 
 
 def cpu_baseline(torch, shape, layer, sample_tokens):
     """fp32 PyTorch oracle on the host cores over the first `sample_tokens` tokens of the same batch."""
     import oracle
+    threads, model = host_cpu()
+    torch.set_num_threads(threads)
     m = min(sample_tokens, layer.M)
     x, logits = layer.x[:m].cpu(), layer.logits[:m].cpu()
     w1, w2 = layer.w1.cpu(), layer.w2.cpu()
@@ -248,11 +315,35 @@ def cpu_baseline(torch, shape, layer, sample_tokens):
     got = layer.out[:m].float().cpu()
     err = (got - ref).abs().max().item()
     return {"value": round(layer_flops(m, shape["H"], shape["F"], shape["topk"]) / dt / 1e12, 4), "unit": "TFLOP/s",
-            "cores": torch.get_num_threads(), "kind": "port",
+            "cores": threads, "kind": "port", "cpu_model": model, "host_cpus": os.cpu_count(),
             "sample": "fp32 PyTorch oracle, first %d tokens of the M=%d batch, weights upcast per expert, 1 rep, %.1f s"
                       % (m, layer.M, dt),
             "us_per_layer_sample": round(dt * 1e6, 0), "max_abs_err_vs_gpu": err,
             "ref_max_abs": ref.abs().max().item()}
+
+
+def oracle_error(torch, shape, layer, tokens=48, fp8=None):
+    """Max-abs error of the layer's last output against the CPU oracle on an evenly spaced sample of tokens."""
+    import oracle
+    layer.fused()
+    torch.cuda.synchronize()
+    M = layer.M
+    idx = torch.arange(M) if M <= tokens else torch.arange(0, M, M // tokens)[:tokens]
+    x, logits = layer.x[idx.cuda()].cpu(), layer.logits[idx.cuda()].cpu()
+    if fp8:
+        # the GPU-prepared codes and scales are bit-identical to the oracle's own (a GPU test holds that):
+        # handing them over saves the CPU from quantising 1.4e9 weights
+        w1q, w1s, w2q, w2s = fp8
+        E, F2, H = w1q.shape
+        wq = (w1q.cpu().numpy().reshape(E * F2, H), w1s.cpu().numpy().reshape(-1),
+              w2q.cpu().numpy().reshape(E * w2q.shape[1], w2q.shape[2]), w2s.cpu().numpy().reshape(-1))
+        ref, _ = oracle.fused_moe_fp8(x, layer.w1.cpu(), layer.w2.cpu(), logits, shape["topk"], True, weights_q=wq)
+    else:
+        ref = oracle.fused_moe(x, layer.w1.cpu(), layer.w2.cpu(), logits, shape["topk"], True)
+    got = layer.out[idx.cuda()].float().cpu()
+    return {"tokens_checked": int(idx.numel()), "max_abs_err": (got - ref).abs().max().item(),
+            "ref_max_abs": ref.abs().max().item(),
+            "rel_frobenius_err": ((got - ref).norm() / ref.norm()).item()}
 
 
 def routing_bench(torch, N, steps, warmup, seed):
@@ -306,6 +397,75 @@ def routing_bench(torch, N, steps, warmup, seed):
     return out
 
 
+def make_weights(torch, shape, seed, dtype=None, scale=0.02):
+    H, F, E = shape["H"], shape["F"], shape["E"]
+    dt = dtype or torch.bfloat16
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    w1 = (torch.randn(E, 2 * F, H, generator=g, device="cuda") * scale).to(dt)
+    w2 = (torch.randn(E, H, F, generator=g, device="cuda") * scale).to(dt)
+    return w1, w2
+
+
+def compact(rec):
+    return {k: rec[k] for k in ("tokens", "us_per_layer", "tflops", "gbps", "bound", "roofline_frac", "block", "split_k")}
+
+
+def other_configs(torch, N, args, mixtral_weights):
+    """Compact records of the workloads the headline does not cover."""
+    out = {}
+    steps, warmup = args.steps, args.warmup
+    # small layer: 176 MB of weights fit the 256 MB Infinity Cache -> flush between repetitions
+    shape = SHAPES["small"]
+    w1, w2 = make_weights(torch, shape, args.seed)
+    rec, layer = measure(torch, N, shape, 64, w1, w2, steps, warmup, args.seed, flush=True)
+    warm, _ = measure(torch, N, shape, 64, w1, w2, steps, warmup, args.seed)
+    out["small"] = dict(compact(rec), stage_us=rec["stage_us"], cache_flush=rec["cache_flush"],
+                        us_per_layer_back_to_back=warm["us_per_layer"], vs_oracle=oracle_error(torch, shape, layer, 64))
+    del w1, w2, layer
+    # routing-only stress: gating + block-aligned sort, bit-exact against the oracle
+    out["routing_stress"] = {"tokens": 65536, "experts": 64, "topk": 6, "bound": "hbm (latency bound in practice)",
+                             "blocks": routing_bench(torch, N, steps, warmup, args.seed)}
+    # fine-grained many-expert layer
+    shape = SHAPES["fine"]
+    w1, w2 = make_weights(torch, shape, args.seed)
+    sweep = []
+    for M in shape["sweep"]:
+        rec, layer = measure(torch, N, shape, M, w1, w2, steps, warmup, args.seed)
+        sweep.append(dict(compact(rec), stage_us=rec["stage_us"]))
+    out["fine"] = {"workload": "H=2048 F=1408 E=64 top-6, Zipf(1.2)-skewed load, bf16", "sweep": sweep,
+                   "vs_oracle_M8192": oracle_error(torch, shape, layer)}
+    del w1, w2, layer
+    # fp8 Mixtral
+    from fast_route_amd import prepare_weights_fp8
+    shape = SHAPES["mixtral"]
+    w1, w2 = mixtral_weights
+    fp8 = prepare_weights_fp8(w1, w2)
+    sweep = []
+    for M in (16, 256, 4096):
+        rec, layer = measure(torch, N, shape, M, w1, w2, steps, warmup, args.seed, fp8)
+        sweep.append(dict(compact(rec), stage_us=rec["stage_us"]))
+    out["fp8"] = {"workload": "Mixtral shape, e4m3 weights (scale per expert and output channel), bf16 activations quantised per token",
+                  "peak_tflops": PEAK_FP8_TFLOPS, "sweep": sweep,
+                  "vs_oracle_M4096": oracle_error(torch, shape, layer, 24, fp8=fp8)}
+    del fp8, layer
+    return out
+
+
+def reference_protocol(torch, N, args):
+    """The reference's own benchmark protocol (benchmarks/fused_route/moe_bench.py:10-38,53,83-99): fp16 operands
+    drawn as randn / 10, shape from -n (ffn) -k (hidden) -e --topk, m = 2^0 .. 2^14, and its "TFLOPS" figure
+    2*m*n*k / t (a sixth of the layer's real work at top-2) next to the real one."""
+    shape = dict(H=args.k, F=args.n, E=args.e, topk=args.topk, zipf=False)
+    w1, w2 = make_weights(torch, shape, args.seed, torch.float16, 0.1)
+    rows = []
+    for m in ([args.tokens] if args.no_sweep else [2 ** i for i in range(15)]):
+        rec, _ = measure(torch, N, shape, m, w1, w2, args.steps, args.warmup, args.seed, dtype=torch.float16, x_scale=0.1)
+        rows.append({"m": m, "us_per_layer": rec["us_per_layer"], "ref_2mnk_tflops": rec["ref_2mnk_tflops"],
+                     "tflops": rec["tflops"], "block": rec["block"]})
+    return {"protocol": "fp16, randn/10, n=%d k=%d e=%d topk=%d, mean of %d back-to-back steps" % (args.n, args.k, args.e, args.topk, args.steps),
+            "ref_2mnk_tflops_is": "2*m*n*k / t, the figure the reference plots (README moe_bench.png)", "rows": rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -317,11 +477,19 @@ def main():
     ap.add_argument("--seed", type=int, default=1337)
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the small / routing / fine-grained / fp8 records")
     ap.add_argument("--cpu-tokens", type=int, default=1024)
     ap.add_argument("--routing", action="store_true", help="also time the routing-only stress workload")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB device copy: the kernel of known size that calibrates "
                          "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc")
+    # the reference's flag names (benchmarks/fused_route/moe_bench.py:10-38)
+    ap.add_argument("-n", type=int, default=8192, help="reference protocol: intermediate (ffn) size")
+    ap.add_argument("-k", type=int, default=4096, help="reference protocol: hidden size")
+    ap.add_argument("-e", type=int, default=16, help="reference protocol: experts")
+    ap.add_argument("--topk", type=int, default=2, help="reference protocol: experts per token")
+    ap.add_argument("--reference-protocol", action="store_true",
+                    help="run the reference's sweep (fp16 randn/10, m = 2^0..2^14 at -n -k -e --topk) instead of the workloads")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X runs the whole layer); --gpus must be 1")
@@ -331,26 +499,29 @@ def main():
     N.lib()
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
     torch.cuda.set_device(0)
+    if args.reference_protocol:
+        print(json.dumps({"metric": "reference_protocol_moe_bench", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                          "dtype": "f16", "data": "synthetic", **reference_protocol(torch, N, args)}))
+        return
     shape = SHAPES[args.shape]
     H, F, E, topk = shape["H"], shape["F"], shape["E"], shape["topk"]
-    g = torch.Generator(device="cuda").manual_seed(args.seed)
-    w1 = (torch.randn(E, 2 * F, H, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
-    w2 = (torch.randn(E, H, F, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    w1, w2 = make_weights(torch, shape, args.seed)
 
     fp8 = None
     sweep_ms = shape["sweep"]
+    flush = 3 * E * F * H * 2 <= (512 << 20)  # weights that could stay in the Infinity Cache between repetitions
     if args.dtype == "fp8":
         from fast_route_amd import prepare_weights_fp8
         fp8 = prepare_weights_fp8(w1, w2)
         sweep_ms = [16, 256, 4096] if args.shape == "mixtral" else shape["sweep"]
-    head, layer = measure(torch, N, shape, args.tokens, w1, w2, args.steps, args.warmup, args.seed, fp8)
+    head, layer = measure(torch, N, shape, args.tokens, w1, w2, args.steps, args.warmup, args.seed, fp8, flush=flush)
     sweep = []
     if not args.no_sweep:
         for M in sweep_ms:
             if M == args.tokens:
                 sweep.append(head)
                 continue
-            rec, _ = measure(torch, N, shape, M, w1, w2, args.steps, args.warmup, args.seed, fp8)
+            rec, _ = measure(torch, N, shape, M, w1, w2, args.steps, args.warmup, args.seed, fp8, flush=flush)
             sweep.append(rec)
     result = {
         "metric": "moe_layer_tflops_%s_%s_M%d" % (args.shape, args.dtype, args.tokens),
@@ -378,6 +549,12 @@ def main():
         result["routing_stress"] = routing_bench(torch, N, args.steps, args.warmup, args.seed)
     if not args.no_cpu and fp8 is None:
         result["cpu_baseline"] = cpu_baseline(torch, shape, layer, args.cpu_tokens)
+    default_run = args.shape == "mixtral" and args.dtype == "bf16" and not args.no_sweep
+    if default_run and not args.no_configs:
+        del layer
+        result["configs"] = other_configs(torch, N, args, (w1, w2))
+        rp_args = argparse.Namespace(**{**vars(args), "no_sweep": True, "tokens": 4096})
+        result["reference_protocol_row"] = reference_protocol(torch, N, rp_args)
     print(json.dumps(result))
 
 

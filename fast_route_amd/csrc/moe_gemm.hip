@@ -152,6 +152,12 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
   a.num_experts = E;
   a.tail_ws = tail_ws;
   a.long_k = 1;
+  if (down_rows_fits(n, F, H, sorted_len, elem_bytes(dtype)) && out_dtype == dtype) {
+    // a handful of pairs: weight rows streamed past the activated rows, routed weight and top-k sum in the same kernel
+    a.out = out;
+    if (dtype == FR_BF16) return launch_down_rows<bf16_t>(a, topk, block, sorted_len, st);
+    return launch_down_rows<f16_t>(a, topk, block, sorted_len, st);
+  }
   if (splits == 1) {
     // one slice: each pair's row in the operands' 2-byte type (bf16 for fp8 operands), half the partial traffic
     int rc = dispatch_dtype<EPI_PLAIN>(a, dtype, block, 1, sorted_len / block * block, st);

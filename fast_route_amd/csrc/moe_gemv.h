@@ -166,4 +166,222 @@ int launch_gateup_rows(const GemmArgs& a, int block, int64_t sorted_len, hipStre
   return check_launch("gateup_rows_kernel");
 }
 
+// ---- down projection + top-k combine for a handful of pairs -------------------------------
+// out[m, h] = sum over the pairs p of token m of topk_w[p] * (act[slot(p), :] . W2[expert(p), h, :]).
+// With at most kDownPairs routed pairs in the whole batch the job is again to stream each active
+// expert's H weight rows once at HBM rate - but these rows are F elements long (28 KB for F = 14336),
+// too long to keep every pair's activated row in LDS next to many resident wavefronts.  So the K range
+// is split over the wavefronts of a workgroup: wavefront w keeps ITS slice (CH chunks of 512 elements)
+// of every pair's activated row in registers for the whole kernel, and for each of the workgroup's output
+// features streams the same slice of the weight row of every active expert (16-byte non-temporal loads,
+// HB features x CH chunks in flight per lane), multiplies with v_dot2 in fp32, sums over its lanes and
+// leaves the partial sums in LDS; after one barrier per HB features a few threads add the wavefronts'
+// partial sums in wavefront order, apply the routed weights, add a token's pairs in slot order and store
+// out[m, h] - no partial buffer, no combine launch, no K slices in HBM; the order of every sum is fixed
+// by the routing arrays, so results are identical from run to run.
+constexpr int kDownPairs = 4;     // routed pairs in the batch, at most (with 8, two weight-row loads per lane and step fit the
+                                  // registers next to the activated rows: measured 10-18 % slower than the tile kernel with K slices)
+constexpr int kDownWaves = 16;    // wavefronts per workgroup, at most
+constexpr int kDownMinK = 4096;   // shorter rows: the tile kernel with K slices is as fast
+
+// CH chunks of 512 elements per wavefront: 1 or 2 (more would spill at 16 wavefronts per CU), the smaller that
+// leaves at most kDownWaves wavefronts, or 0: rows of up to 16384 elements
+inline int down_rows_chunks(int64_t K) {
+  if (K % 512 != 0) return 0;
+  const int64_t nc = K / 512;
+  for (int ch = 1; ch <= 2; ++ch)
+    if (nc % ch == 0 && nc / ch <= kDownWaves) return ch;
+  return 0;
+}
+inline bool down_rows_fits(int64_t n_pairs, int64_t K, int64_t N, int64_t sorted_len, int elem_bytes) {
+  return elem_bytes == 2 && n_pairs >= 1 && n_pairs <= kDownPairs && K >= kDownMinK && down_rows_chunks(K) != 0 &&
+         N % 8 == 0 && sorted_len <= 4096;
+}
+
+// NP = pairs the registers are sized for (>= the batch's), HB = output features per step.
+// a.X = act [slots, K], a.W = W2 [E, N, K], a.out = out [tokens, N]; a.group_t = routing block;
+// `slots` = whole routing blocks inside sorted_token_ids; hpw = features per workgroup (multiple of HB).
+//
+// Every wavefront builds the pair table for itself (no LDS, no barrier before the first weight load):
+// the real slots in order, kept one pair per LANE of a few registers and read back with v_readlane;
+// pairs of one expert are adjacent (the routing arrays are sorted by expert), a run of them is a group.
+// The weight stream is a sequence of steps (round of HB features, group); the loads of step i + 1 are in
+// flight while step i is multiplied (two register buffers), so the stream never drains inside a workgroup.
+template <typename T, int CH, int NP, int HB>
+__global__ void __launch_bounds__(kDownWaves * kWave) down_rows_kernel(GemmArgs a, int topk, int slots, int hpw) {
+  __shared__ float red[2][kDownWaves][HB * NP];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
+  const int block = a.group_t;
+  // ---- pair table ------------------------------------------------------------------------------
+  int t_slot = 0, t_sid = 0, t_exp = 0, g_first = 0;  // lane p: pair p; lane g: first pair of group g
+  int np = 0, ng = 0;
+  {
+    const int npost = *a.npost;
+    int prev_e = -1;
+    for (int base = 0; base < slots; base += kWave) {
+      const int s = base + lane;
+      int sid = a.num_valid, ev = 0;
+      if (s < slots) {
+        sid = a.sorted[s];
+        ev = a.expert_ids[s / block];
+      }
+      unsigned long long m = __ballot(s < npost && sid < a.num_valid);
+      while (m != 0 && np < NP) {
+        const int bpos = __builtin_ctzll(m);
+        m &= m - 1;
+        const int e = __builtin_amdgcn_readlane(ev, bpos);
+        t_slot = (lane == np ? (base + bpos) : t_slot);
+        t_sid = (lane == np ? (__builtin_amdgcn_readlane(sid, bpos)) : t_sid);
+        t_exp = (lane == np ? (e) : t_exp);
+        if (e != prev_e) {
+          g_first = (lane == ng ? (np) : g_first);
+          ++ng;
+          prev_e = e;
+        }
+        ++np;
+      }
+      if (base + kWave >= npost) break;
+    }
+    g_first = (lane == ng ? (np) : g_first);  // group g = pairs [g_first[g], g_first[g + 1])
+  }
+  const float t_w = lane < np ? a.topk_w[t_sid] : 0.f;
+  const int t_tok = t_sid / topk;
+  const int tokens = a.num_valid / topk;
+  // ---- this wavefront's slice of every pair's activated row -----------------------------------
+  const int kofs = (wave * CH) * 512 + lane * 8;  // first element of the lane's first chunk
+  u32x4 ar[NP][CH];
+#pragma unroll
+  for (int p = 0; p < NP; ++p)
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      ar[p][c] = u32x4{0u, 0u, 0u, 0u};
+      if (p < np)
+        ar[p][c] = *reinterpret_cast<const u32x4*>(static_cast<const T*>(a.X) +
+                                                   static_cast<int64_t>(__builtin_amdgcn_readlane(t_slot, p)) * a.ldx + kofs + c * 512);
+    }
+  const int h_begin = blockIdx.x * hpw, h_end = min(h_begin + hpw, a.N);
+  const int rounds = (h_end - h_begin + HB - 1) / HB, steps = rounds * ng;
+  float acc[HB][NP];
+#pragma unroll
+  for (int hb = 0; hb < HB; ++hb)
+#pragma unroll
+    for (int p = 0; p < NP; ++p) acc[hb][p] = 0.f;
+  u32x4 w0[HB][CH], w1[HB][CH];
+  // loads of step (round r, group g) into wb
+#define FR_DR_ISSUE(wb, r_, g_)                                                                                   \
+  {                                                                                                               \
+    const int e_ = __builtin_amdgcn_readlane(t_exp, __builtin_amdgcn_readlane(g_first, (g_)));                    \
+    const T* wp_ = static_cast<const T*>(a.W) + static_cast<int64_t>(e_) * a.w_expert_stride + kofs;              \
+    _Pragma("unroll") for (int hb = 0; hb < HB; ++hb) {                                                           \
+      const int h_ = h_begin + (r_) * HB + hb < a.N ? h_begin + (r_) * HB + hb : a.N - 1;                         \
+      _Pragma("unroll") for (int c = 0; c < CH; ++c)                                                              \
+        wb[hb][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp_ + static_cast<int64_t>(h_) * a.ldw + c * 512)); \
+    }                                                                                                             \
+  }
+  // step (round r, group g) multiplied from wb
+#define FR_DR_FMA(wb, g_)                                                                                         \
+  {                                                                                                               \
+    const int p0_ = __builtin_amdgcn_readlane(g_first, (g_)), p1_ = __builtin_amdgcn_readlane(g_first, (g_) + 1); \
+    _Pragma("unroll") for (int p = 0; p < NP; ++p) {                                                              \
+      if (p >= p0_ && p < p1_) {                                                                                  \
+        _Pragma("unroll") for (int hb = 0; hb < HB; ++hb)                                                         \
+          _Pragma("unroll") for (int c = 0; c < CH; ++c)                                                          \
+            _Pragma("unroll") for (int d = 0; d < 4; ++d) acc[hb][p] = Dot2<T>::fma2(wb[hb][c][d], ar[p][c][d], acc[hb][p]); \
+      }                                                                                                           \
+    }                                                                                                             \
+  }
+  // after a round's last group the round is summed over lanes, wavefronts and a token's pairs, and stored
+#define FR_DR_FINISH(r_, g_)                                                                                      \
+  {                                                                                                               \
+    if ((g_) == ng - 1) {                                                                                         \
+      const int buf_ = (r_) & 1, h0_ = h_begin + (r_) * HB;                                                       \
+      _Pragma("unroll") for (int hb = 0; hb < HB; ++hb)                                                           \
+        _Pragma("unroll") for (int p = 0; p < NP; ++p) {                                                          \
+          if (p < np) {                                                                                           \
+            const float v_ = wave_sum(acc[hb][p]);                                                                \
+            if (lane == 0) red[buf_][wave][hb * NP + p] = v_;                                                     \
+          }                                                                                                       \
+          acc[hb][p] = 0.f;                                                                                       \
+        }                                                                                                         \
+      __syncthreads(); /* one barrier per round: the other buffer is written only after every wavefront passed this one */ \
+      if (threadIdx.x < HB * tokens) {                                                                            \
+        const int hb = threadIdx.x % HB, m = threadIdx.x / HB, h = h0_ + hb;                                      \
+        if (h < h_end) {                                                                                          \
+          float s_ = 0.f;                                                                                         \
+          for (int p = 0; p < np; ++p) { /* wavefronts in order, then the token's pairs in slot order */          \
+            if (__builtin_amdgcn_readlane(t_tok, p) != m) continue;                                               \
+            float d_ = 0.f;                                                                                       \
+            for (int wv = 0; wv < nwaves; ++wv) d_ += red[buf_][wv][hb * NP + p];                                 \
+            s_ += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(t_w), p)) * d_;                         \
+          }                                                                                                       \
+          static_cast<typename Elem<T>::out_t*>(a.out)[static_cast<int64_t>(m) * a.ldo + h] = static_cast<typename Elem<T>::out_t>(s_); \
+        }                                                                                                         \
+      }                                                                                                           \
+    }                                                                                                             \
+  }
+#define FR_DR_NEXT(r_, g_) { if (++(g_) == ng) { (g_) = 0; ++(r_); } }
+  // a buffer is refilled as soon as its step has been multiplied, before that round's sums: two steps' loads stay in flight
+  int r = 0, g = 0, rn = 0, gn = 0;  // step being multiplied, step being loaded
+  if (steps > 0) {
+    FR_DR_ISSUE(w0, rn, gn)
+    FR_DR_NEXT(rn, gn)
+  }
+  if (steps > 1) {
+    FR_DR_ISSUE(w1, rn, gn)
+    FR_DR_NEXT(rn, gn)
+  }
+  for (int i = 0; i < steps; i += 2) {
+    FR_DR_FMA(w0, g)
+    if (i + 2 < steps) {
+      FR_DR_ISSUE(w0, rn, gn)
+      FR_DR_NEXT(rn, gn)
+    }
+    FR_DR_FINISH(r, g)
+    FR_DR_NEXT(r, g)
+    if (i + 1 >= steps) break;
+    FR_DR_FMA(w1, g)
+    if (i + 3 < steps) {
+      FR_DR_ISSUE(w1, rn, gn)
+      FR_DR_NEXT(rn, gn)
+    }
+    FR_DR_FINISH(r, g)
+    FR_DR_NEXT(r, g)
+  }
+#undef FR_DR_NEXT
+#undef FR_DR_FINISH
+#undef FR_DR_FMA
+#undef FR_DR_ISSUE
+}
+
+template <typename T, int CH>
+int launch_down_rows_ch(const GemmArgs& a, int topk, int block, int64_t sorted_len, hipStream_t st) {
+  const int nwaves = static_cast<int>(a.K / 512 / CH);
+  const int np = a.num_valid;
+  GemmArgs b = a;
+  b.group_t = block;
+  const int slots = static_cast<int>(sorted_len / block * block);
+  // one workgroup per CU (its wavefronts fill the CU's registers with the activated rows and the two
+  // weight buffers: 16 loads of 16 bytes in flight per lane), steps of HB features
+  auto go = [&](auto kern, int HB) {
+    int hpw = static_cast<int>(ceil_div(a.N, 256));
+    hpw = static_cast<int>(round_up(hpw < HB ? HB : hpw, HB));
+    const unsigned grid = static_cast<unsigned>(ceil_div(a.N, hpw));
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(nwaves * kWave), 0, st, b, topk, slots, hpw);
+  };
+  constexpr int HB = 8 / CH;
+  static_assert(kDownPairs == 4, "register variants below");
+  if (np <= 2) go(down_rows_kernel<T, CH, 2, HB>, HB);
+  else go(down_rows_kernel<T, CH, 4, HB>, HB);
+  return check_launch("down_rows_kernel");
+}
+
+template <typename T>
+int launch_down_rows(const GemmArgs& a, int topk, int block, int64_t sorted_len, hipStream_t st) {
+  switch (down_rows_chunks(a.K)) {
+    case 1: return launch_down_rows_ch<T, 1>(a, topk, block, sorted_len, st);
+    case 2: return launch_down_rows_ch<T, 2>(a, topk, block, sorted_len, st);
+    default: return fail(FR_E_SHAPE, "down projection by rows: K=%d", a.K);
+  }
+}
+
 }  // namespace fr

@@ -556,6 +556,33 @@ def test_reference_end_to_end_recipe(native, m):
     torch.testing.assert_close(out.float().cpu(), want, atol=1e-2, rtol=0)
 
 
+@pytest.mark.parametrize("E,k,H,Fd", [(8, 2, 256, 4096), (8, 2, 512, 5120), (16, 6, 256, 4096), (8, 8, 128, 8192),
+                                      (4, 1, 384, 14336), (64, 6, 256, 16384)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_decode_down_projection_by_rows(native, E, k, H, Fd, dtype):
+    """At most 4 routed pairs and weight rows of 4096..16384 elements (multiples of 512): the down
+    projection streams weight rows past the activated rows and sums a token's pairs itself - no partial
+    buffer, no combine launch.  Token counts on both sides of that limit (up to 8 pairs), against the
+    oracle; the same bits on every run."""
+    from fast_route_amd import fused_moe, fused_experts
+    for M in range(1, 8 // k + 1):
+        _say(f"down by rows E={E} k={k} H={H} F={Fd} {dtype} M={M}")
+        x, logits, w1, w2 = _inputs(M, H, Fd, E, 77 + M, dtype)
+        xd, w1d, w2d, ld = x.cuda(), w1.cuda(), w2.cuda(), logits.cuda()
+        out = fused_moe(xd, w1d, w2d, ld, k, True)
+        torch.cuda.synchronize()
+        _assert_close(out, oracle.fused_moe(x, w1, w2, logits, k, True), dtype, f"down by rows M={M}")
+        for _ in range(3):
+            assert torch.equal(fused_moe(xd, w1d, w2d, ld, k, True), out)
+    if k == 2 and E >= 4:
+        _say("down by rows: a token naming one expert twice, another token sharing it")
+        ids = torch.tensor([[3, 3], [3, 1], [0, 2]], dtype=torch.int32)
+        wts = torch.tensor([[0.25, 0.5], [0.7, 0.3], [0.9, 0.1]])
+        x, _, w1, w2 = _inputs(3, H, Fd, E, 5, dtype)
+        out = fused_experts(x.cuda(), w1.cuda(), w2.cuda(), wts.cuda(), ids.cuda())
+        _assert_close(out, oracle.moe_experts(x, w1, w2, wts, ids), dtype, "down by rows, repeated expert")
+
+
 def test_random_shapes_against_oracle(native):
     """Forty seeded random layer shapes (token count, widths, expert count, top-k, dtype, renormalisation)
     against the oracle: every plan boundary gets neighbours on both sides sooner or later."""
