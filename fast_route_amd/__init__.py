@@ -10,6 +10,7 @@ from .layers.fused_moe import fused_moe, fused_experts  # noqa: F401
 from .layers.fp8 import fused_moe_fp8, prepare_weights_fp8, quantize_rows_e4m3  # noqa: F401
 from .ops.fused_moe import moe_align_block_size, invoke_fused_moe_kernel  # noqa: F401
 from .ops.stable_route import fused_route, topk_softmax  # noqa: F401
+from .tuning import get_tunables, prepare, reset_tunables, set_tunables, tunables  # noqa: F401
 
 __all__ = [
     "fused_moe",
@@ -21,4 +22,9 @@ __all__ = [
     "invoke_fused_moe_kernel",
     "fused_route",
     "topk_softmax",
+    "set_tunables",
+    "get_tunables",
+    "reset_tunables",
+    "tunables",
+    "prepare",
 ]

@@ -18,6 +18,10 @@ class FrMoePlan(ctypes.Structure):
                 ("workspace_bytes", c_int64), ("tail_bytes", c_int64)]
 
 
+class FrMoeTunables(ctypes.Structure):
+    _fields_ = [("block", c_int32), ("split_k", c_int32), ("group_m", c_int32), ("no_tail_split", c_int32)]
+
+
 # name -> (restype, argtypes); must list every symbol the header declares
 SIGNATURES = {
     "fr_version": (c_int, []),
@@ -28,6 +32,9 @@ SIGNATURES = {
     "fr_moe_align": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "fr_moe_grouped_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                     c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "fr_moe_prepare": (c_int, [c_int]),
+    "fr_moe_set_tunables": (c_int, [ctypes.POINTER(FrMoeTunables)]),
+    "fr_moe_get_tunables": (c_int, [ctypes.POINTER(FrMoeTunables)]),
     "fr_moe_get_plan": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, c_int, ctypes.POINTER(FrMoePlan)]),
     "fr_moe_gateup_silu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                    c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),

@@ -22,6 +22,9 @@ int64_t tail_scratch_bytes(int block, int dtype, int64_t K, int64_t N, bool gate
 int quant_rows(const void* x, int dtype, int64_t rows, const int32_t* rows_dev, int64_t K, int64_t ldx, void* q_out,
                float* scale_out, hipStream_t st);
 
+// the study knobs set through fr_moe_set_tunables (all zero: the library decides)
+const fr_moe_tunables& tunables();
+
 // gating + routing arrays in one launch (small batches); see routing.hip
 bool route_align_fits(int64_t M, int E, int topk);
 int route_align_small(const void* logits, int logits_dtype, int64_t M, int E, int topk, int renorm, int block,

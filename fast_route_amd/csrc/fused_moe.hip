@@ -56,6 +56,8 @@ Carve carve(void* base, int64_t M, int64_t H, int64_t F, int E, int topk, int dt
   return c;
 }
 
+fr_moe_tunables g_tunables = {0, 0, 0, 0};
+
 int check_layer_shapes(const char* who, int64_t M, int64_t H, int64_t F, int E, int topk, int dtype) {
   FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16 || dtype == FR_FP8_E4M3, FR_E_DTYPE, "%s: dtype %d not in {f16, bf16, fp8_e4m3}", who, dtype);
   FR_REQUIRE(M >= 0 && H > 0 && F > 0, FR_E_SHAPE, "%s: M=%lld H=%lld F=%lld", who, (long long)M, (long long)H, (long long)F);
@@ -67,9 +69,30 @@ int check_layer_shapes(const char* who, int64_t M, int64_t H, int64_t F, int E, 
 }
 
 }  // namespace
+const fr_moe_tunables& tunables() { return g_tunables; }
 }  // namespace fr
 
 using namespace fr;
+
+extern "C" int fr_moe_set_tunables(const fr_moe_tunables* t) {
+  if (!t) {
+    g_tunables = fr_moe_tunables{0, 0, 0, 0};
+    return FR_OK;
+  }
+  FR_REQUIRE(t->block == 0 || t->block == 16 || t->block == 32 || t->block == 64 || t->block == 128 || t->block == 256,
+             FR_E_SHAPE, "fr_moe_set_tunables: block=%d not in {0, 16, 32, 64, 128, 256}", t->block);
+  FR_REQUIRE(t->split_k >= 0 && t->split_k <= 64, FR_E_SHAPE, "fr_moe_set_tunables: split_k=%d outside [0, 64]", t->split_k);
+  FR_REQUIRE(t->group_m >= 0 && t->group_m <= 64, FR_E_SHAPE, "fr_moe_set_tunables: group_m=%d outside [0, 64]", t->group_m);
+  FR_REQUIRE(t->no_tail_split == 0 || t->no_tail_split == 1, FR_E_SHAPE, "fr_moe_set_tunables: no_tail_split=%d", t->no_tail_split);
+  g_tunables = *t;
+  return FR_OK;
+}
+
+extern "C" int fr_moe_get_tunables(fr_moe_tunables* t) {
+  FR_REQUIRE(t, FR_E_NULL, "fr_moe_get_tunables: null pointer");
+  *t = g_tunables;
+  return FR_OK;
+}
 
 extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk, int dtype, fr_moe_plan* plan) {
   FR_REQUIRE(plan, FR_E_NULL, "fr_moe_get_plan: null plan");
@@ -94,6 +117,7 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   else if (avg < 52 && H >= 4096) block = 64;
   else if (avg < t256) block = 128;
   else block = 256;
+  if (g_tunables.block) block = g_tunables.block;
   // Down projection: N = H gives few feature tiles, so K is split.
   const int bf = block == 16 ? 64 : (block == 32 ? 128 : 256);
   const int64_t blocks = n <= E ? n : (block >= 128 ? ceil_div(n, block) + E / 2 : E);
@@ -132,10 +156,16 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
     if (n <= E && 2 * n > E && tiles <= 512)
       while (split < 4 && F / (split * 2) >= 8 * bk_elems) split *= 2;
   }
+  int64_t tail_bytes = tail_up > tail_down ? tail_up : tail_down;
+  if (g_tunables.split_k) {  // as many slices as asked for, as far as every slice keeps 8 K tiles
+    split = g_tunables.split_k;
+    while (split > 1 && F / split < 8 * bk_elems) --split;
+  }
+  if (g_tunables.no_tail_split) tail_bytes = 0;
   plan->block = block;
   plan->split_k = split;
   plan->sorted_len = n + static_cast<int64_t>(E) * (block - 1);
-  plan->tail_bytes = tail_up > tail_down ? tail_up : tail_down;
+  plan->tail_bytes = tail_bytes;
   plan->workspace_bytes = carve(nullptr, M, H, F, E, topk, dtype, *plan).total;
   return FR_OK;
 }

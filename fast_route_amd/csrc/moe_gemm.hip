@@ -34,7 +34,10 @@ __global__ __launch_bounds__(256) void combine_kernel(const P* __restrict__ part
 #define FR_DECLARE_TILES(T)                                                                       \
   extern template int dispatch_block<T, EPI_PLAIN>(GemmArgs, int, int, int64_t, hipStream_t);     \
   extern template int dispatch_block<T, EPI_SILU>(GemmArgs, int, int, int64_t, hipStream_t);      \
-  extern template int dispatch_block<T, EPI_DOWN>(GemmArgs, int, int, int64_t, hipStream_t);
+  extern template int dispatch_block<T, EPI_DOWN>(GemmArgs, int, int, int64_t, hipStream_t);      \
+  extern template int prepare_tiles<T, EPI_PLAIN>();                                              \
+  extern template int prepare_tiles<T, EPI_SILU>();                                               \
+  extern template int prepare_tiles<T, EPI_DOWN>();
 FR_DECLARE_TILES(bf16_t)
 FR_DECLARE_TILES(f16_t)
 FR_DECLARE_TILES(fp8_t)
@@ -236,4 +239,25 @@ extern "C" int fr_moe_down_combine_fp8(const void* actq, const float* act_scale,
   return down_impl(actq, act_scale, w2q, w2_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, M,
                    H, F, E, topk, block, split_k, FR_FP8_E4M3, out_dtype, partial, out, static_cast<float*>(tail_ws),
                    static_cast<hipStream_t>(stream), "fr_moe_down_combine_fp8");
+}
+
+// Every kernel the grouped GEMM entry points can launch for `dtype`, set up on the current device.
+extern "C" int fr_moe_prepare(int dtype) {
+  int rc;
+  if (dtype == FR_BF16) {
+    rc = prepare_tiles<bf16_t, EPI_PLAIN>();
+    if (rc == FR_OK) rc = prepare_tiles<bf16_t, EPI_SILU>();
+    if (rc == FR_OK) rc = prepare_tiles<bf16_t, EPI_DOWN>();
+  } else if (dtype == FR_F16) {
+    rc = prepare_tiles<f16_t, EPI_PLAIN>();
+    if (rc == FR_OK) rc = prepare_tiles<f16_t, EPI_SILU>();
+    if (rc == FR_OK) rc = prepare_tiles<f16_t, EPI_DOWN>();
+  } else if (dtype == FR_FP8_E4M3) {
+    rc = prepare_tiles<fp8_t, EPI_PLAIN>();
+    if (rc == FR_OK) rc = prepare_tiles<fp8_t, EPI_SILU>();
+    if (rc == FR_OK) rc = prepare_tiles<fp8_t, EPI_DOWN>();
+  } else {
+    return fail(FR_E_DTYPE, "fr_moe_prepare: dtype %d not in {f16, bf16, fp8_e4m3}", dtype);
+  }
+  return rc;
 }

@@ -3,4 +3,5 @@
 
 namespace fr {
 template int dispatch_block<bf16_t, EPI_PLAIN>(GemmArgs, int, int, int64_t, hipStream_t);
+template int prepare_tiles<bf16_t, EPI_PLAIN>();
 }  // namespace fr

@@ -3,4 +3,5 @@
 
 namespace fr {
 template int dispatch_block<bf16_t, EPI_SILU>(GemmArgs, int, int, int64_t, hipStream_t);
+template int prepare_tiles<bf16_t, EPI_SILU>();
 }  // namespace fr

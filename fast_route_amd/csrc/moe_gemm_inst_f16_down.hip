@@ -3,4 +3,5 @@
 
 namespace fr {
 template int dispatch_block<f16_t, EPI_DOWN>(GemmArgs, int, int, int64_t, hipStream_t);
+template int prepare_tiles<f16_t, EPI_DOWN>();
 }  // namespace fr

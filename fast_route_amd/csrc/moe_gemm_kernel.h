@@ -60,6 +60,7 @@ struct GemmArgs {
   int num_experts;      // E (persistent form: walk order by expert)
   int long_k;           // down projection (few feature tiles, long K): hint for the 128-row tile's form
   float* tail_ws;       // persistent form only: slice buffers for splitting the last round of tiles along K, or nullptr
+  int setup_only;       // do the per-device set-up of the kernel a launch would take (LDS limit, occupancy) and launch nothing
 };
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -620,13 +621,20 @@ _Pragma("unroll") \
 
 template <typename T, typename C, int EPI>
 int launch_gemm(const GemmArgs& a, int splits, hipStream_t st) {
-  static bool attr_set = false;
-  if (C::LDS_BYTES > 65536 && !attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_kernel<T, C, EPI>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess) return fail(FR_E_LAUNCH, "hipFuncSetAttribute(%d B LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
-    attr_set = true;
+  if (C::LDS_BYTES > 65536) {  // the dynamic LDS limit is a property of the kernel on ONE device
+    constexpr int kMaxDevices = 64;
+    static bool attr_set[kMaxDevices] = {};  // a race between threads sets the same attribute twice
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(FR_E_LAUNCH, "grouped GEMM: device %d (%s)", dev, hipGetErrorString(e));
+    if (!attr_set[dev]) {
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_kernel<T, C, EPI>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+      if (e != hipSuccess) return fail(FR_E_LAUNCH, "hipFuncSetAttribute(%d B LDS): %s", C::LDS_BYTES, hipGetErrorString(e));
+      attr_set[dev] = true;
+    }
   }
+  if (a.setup_only) return FR_OK;
   if (C::STAGES > 0) {  // the ring loads address rows by 32-bit byte offsets
     const int64_t x_rows = a.top_k > 0 ? a.num_valid / a.top_k : C::BT;
     const int64_t w_rows = EPI == EPI_SILU ? 2 * static_cast<int64_t>(a.N) : a.N;

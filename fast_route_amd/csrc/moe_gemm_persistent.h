@@ -563,6 +563,11 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
   GemmArgs a = a_in;
   constexpr int BK = C::BKB / static_cast<int>(sizeof(T));
   const int last_k = a.K - (splits - 1) * a.k_per_split;  // K range of the last split
+  if (a.setup_only) {  // both forms a launch may take
+    int resident = 0;
+    const int rc = persistent_grid<T, C, EPI>(&resident);
+    return rc != FR_OK ? rc : launch_gemm<T, C, EPI>(a, splits, st);
+  }
   if (a.k_per_split / BK < C::STAGES + 2 || last_k / BK < C::STAGES + 2 || a.num_experts < 1 || a.num_experts > kMaxExperts) {
     a.tail_ws = nullptr;
     return launch_gemm<T, C, EPI>(a, splits, st);
@@ -573,7 +578,8 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
   if (x_rows * a.ldx * es >= lim || w_rows * a.ldw * es >= lim)
     return fail(FR_E_SHAPE, "token rows (%lld x %lld) or one expert's weights (%lld x %lld) span 4 GiB or more",
                 (long long)x_rows, (long long)a.ldx, (long long)w_rows, (long long)a.ldw);
-  a.group_t = kChunkBlocks;
+  a.group_t = tunables().group_m ? tunables().group_m : kChunkBlocks;
+  if (tunables().no_tail_split) a.tail_ws = nullptr;
   int resident = 0;
   const int rc = persistent_grid<T, C, EPI>(&resident);
   if (rc != FR_OK) return rc;

@@ -54,7 +54,7 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
     a.num_t_blocks = static_cast<int>(ceil_div(sorted_len, BT));
     const int fper = (EPI == EPI_SILU) ? BF / 2 : BF;
     a.num_f_tiles = static_cast<int>(ceil_div(a.N, fper));
-    a.group_t = BT >= 64 ? 4 : 8;
+    a.group_t = tunables().group_m ? tunables().group_m : (BT >= 64 ? 4 : 8);
     a.k_per_split = static_cast<int>(round_up(ceil_div(a.K, splits), bk));
   };
   switch (block) {
@@ -101,6 +101,27 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       return launch_gemm<T, typename TL::T16, EPI>(a, splits, st);
     default: return fail(FR_E_SHAPE, "routing block %d not in {16, 32, 64, 128, 256}", block);
   }
+}
+
+// Per-device set-up (dynamic LDS limits, occupancy queries) of every kernel dispatch_block<T, EPI> can launch,
+// so that no later call has anything left to set up - e.g. a first call under graph capture.
+template <typename T, int EPI>
+int prepare_tiles() {
+  typedef Tiles<T> TL;
+  GemmArgs a = {};
+  a.setup_only = 1;
+  int rc = launch_gemm_persistent<T, typename TL::T256, EPI>(a, 1, nullptr);
+  if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T128P, EPI>(a, 1, nullptr);
+  if (rc == FR_OK) rc = launch_gemm<T, typename TL::T128, EPI>(a, 1, nullptr);
+  if (rc == FR_OK) rc = launch_gemm<T, typename TL::T64, EPI>(a, 1, nullptr);
+  if (rc == FR_OK) rc = launch_gemm<T, typename TL::T32, EPI>(a, 1, nullptr);
+  if (rc == FR_OK) rc = launch_gemm<T, typename TL::T16, EPI>(a, 1, nullptr);
+  if constexpr (EPI == EPI_SILU) {
+    if (rc == FR_OK) rc = launch_gemm<T, typename TL::T64U, EPI>(a, 1, nullptr);
+    if (rc == FR_OK) rc = launch_gemm<T, typename TL::T32L, EPI>(a, 1, nullptr);
+    if (rc == FR_OK) rc = launch_gemm<T, typename TL::T16L, EPI>(a, 1, nullptr);
+  }
+  return rc;
 }
 
 }  // namespace fr

@@ -108,6 +108,37 @@ typedef struct fr_moe_plan {
 } fr_moe_plan;
 int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk, int dtype, fr_moe_plan* plan);
 
+/* Per-device set-up of every grouped-GEMM kernel of `dtype` (FR_F16, FR_BF16, FR_FP8_E4M3) on the
+ * CURRENT device: raises the kernels' dynamic-LDS limits and caches the persistent kernels'
+ * occupancy.  The first call of each tile configuration does the same work lazily; a caller whose
+ * first call would be under graph capture (set-up calls are not stream work) calls this once per
+ * device and dtype beforehand.  Launches nothing.  No counterpart in the reference (Triton compiles
+ * and configures its kernels on first use, fast_route/fast_route/layers/stable_route.py:67). */
+int fr_moe_prepare(int dtype);
+
+/* Study knobs of the tile plan, process-wide (set them from one thread while no call is in
+ * flight; they are read when a call is made, not when its kernels run).  0 in a field leaves
+ * that choice to the library.
+ *   block      routing block = token rows per GEMM tile: 16, 32, 64, 128 or 256
+ *   split_k    K slices of the down projection, 1..64 (1 also switches the last-round split on
+ *              where the tile supports it, as the plan itself would)
+ *   group_m    token blocks walked together over the feature tiles (L2 sharing of weight tiles),
+ *              1..64
+ *   no_tail_split  1: never split the last, partly filled round of tiles along K
+ * fr_moe_get_plan, fr_fused_moe, fr_fused_experts, fr_fused_moe_fp8 and the staged GEMM entry
+ * points all see them.  fr_moe_set_tunables(NULL) restores the defaults.
+ * Replaces: the per-GEMM config dictionaries edited by hand in the reference's tile study
+ * (block_m / group_m / split_k; block_n and block_k are fixed per block size on this hardware),
+ * fast_route/benchmarks/swizzle_moe/v1_moe_fused.py:311-344. */
+typedef struct fr_moe_tunables {
+  int32_t block;
+  int32_t split_k;
+  int32_t group_m;
+  int32_t no_tail_split;
+} fr_moe_tunables;
+int fr_moe_set_tunables(const fr_moe_tunables* t);
+int fr_moe_get_tunables(fr_moe_tunables* t);
+
 /* act[s, :] = silu(x[t] @ W1[e, :F]^T) * (x[t] @ W1[e, F:]^T) for every sorted
  * slot s < num_tokens_post_pad that holds a pair (t = sorted_token_ids[s] / topk),
  * written at row s of act[sorted_len, F].  Rows of padding slots are unspecified

@@ -118,7 +118,8 @@ def test_bench_refuses_more_than_one_gpu():
 
 
 def test_recorded_traffic_matches_profiles_file():
-    """bench.py reports roofline.traffic from profiles/hbm_traffic.json for the workloads recorded there."""
+    """bench.py reports roofline.traffic from profiles/hbm_traffic.json for the workloads recorded there,
+    as long as the kernel sources are the ones the record was measured with."""
     import importlib.util
     import json
     import os
@@ -128,5 +129,43 @@ def test_recorded_traffic_matches_profiles_file():
     spec.loader.exec_module(mod)
     rec = json.load(open(os.path.join(root, "profiles", "hbm_traffic.json")))
     key = "moe_layer_tflops_mixtral_bf16_M4096"
-    assert mod.recorded_traffic(key) == rec[key]["traffic_bytes"] == rec[key]["fetch_bytes"] + rec[key]["write_bytes"]
+    assert rec[key]["traffic_bytes"] == rec[key]["fetch_bytes"] + rec[key]["write_bytes"]
+    # the record counts only for the kernel sources it was measured with
+    want = rec[key]["traffic_bytes"] if rec.get("kernel_sources_sha") == mod.kernel_sources_sha() else None
+    assert mod.recorded_traffic(key) == want
     assert mod.recorded_traffic("no_such_workload") is None
+
+
+def test_tunables_override_the_plan_and_reset():
+    """fr_moe_set_tunables is host logic: the plan follows the overrides, rejects values outside its ranges,
+    and NULL restores the library's own choices."""
+    import fast_route_amd as fr
+    from fast_route_amd import _native
+    lib = _native.lib()
+
+    def plan(M):
+        p = _native.FrMoePlan()
+        assert lib.fr_moe_get_plan(M, 4096, 14336, 8, 2, _native.FR_BF16, p) == 0
+        return p
+
+    base = plan(4096)
+    assert (base.block, base.split_k) == (256, 1) and base.tail_bytes > 0
+    try:
+        fr.set_tunables(block=128, split_k=3)
+        p = plan(4096)
+        assert (p.block, p.split_k) == (128, 3) and p.sorted_len == 8192 + 8 * 127
+        assert fr.get_tunables() == {"block": 128, "split_k": 3, "group_m": 0, "no_tail_split": False}
+        with fr.tunables(no_tail_split=True):
+            assert plan(4096).tail_bytes == 0 and plan(4096).block == 256  # the context replaces, then restores
+        assert plan(4096).block == 128
+        fr.set_tunables(split_k=64)  # as many slices as keep 8 K tiles each: 14336 / (8 * 64) = 28
+        assert plan(4096).split_k == 28
+        with pytest.raises(AssertionError):
+            fr.set_tunables(block=48)
+        with pytest.raises(AssertionError):
+            fr.set_tunables(group_m=65)
+    finally:
+        fr.reset_tunables()
+    p = plan(4096)
+    assert (p.block, p.split_k, p.tail_bytes) == (base.block, base.split_k, base.tail_bytes)
+    assert lib.fr_moe_prepare(_native.FR_F32) == -3

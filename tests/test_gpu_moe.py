@@ -583,6 +583,35 @@ def test_decode_down_projection_by_rows(native, E, k, H, Fd, dtype):
         _assert_close(out, oracle.moe_experts(x, w1, w2, wts, ids), dtype, "down by rows, repeated expert")
 
 
+def test_tunables_and_prepare(native):
+    """Plan overrides (routing block, K slices, walk group, no last-round split) change the kernels a layer takes,
+    never its result beyond fp32 summation order; fr_moe_prepare sets every kernel up without launching."""
+    import fast_route_amd as fr
+    from fast_route_amd import fused_moe
+    dtype = torch.bfloat16
+    fr.prepare(dtype)
+    fr.prepare(torch.float16)
+    fr.prepare("fp8")
+    torch.cuda.synchronize()
+    x, logits, w1, w2 = _inputs(300, 512, 1024, 8, 21, dtype)
+    xd, w1d, w2d, ld = x.cuda(), w1.cuda(), w2.cuda(), logits.cuda()
+    ref = oracle.fused_moe(x, w1, w2, logits, 2, True)
+    base = fused_moe(xd, w1d, w2d, ld, 2, True)
+    _assert_close(base, ref, dtype, "library plan")
+    try:
+        for kw in ({"block": 16}, {"block": 32, "split_k": 3}, {"block": 64, "group_m": 1}, {"block": 128, "split_k": 2},
+                   {"block": 256, "no_tail_split": True}, {"block": 256, "group_m": 3}, {"split_k": 4}, {"group_m": 64}):
+            _say(f"tunables {kw}")
+            with fr.tunables(**kw):
+                out = fused_moe(xd, w1d, w2d, ld, 2, True)
+            torch.cuda.synchronize()
+            _assert_close(out, ref, dtype, f"tunables {kw}")
+            assert (out.float() - base.float()).abs().max() <= 2.0 ** -7 * ref.abs().max()
+    finally:
+        fr.reset_tunables()
+    assert torch.equal(fused_moe(xd, w1d, w2d, ld, 2, True), base)
+
+
 def test_random_shapes_against_oracle(native):
     """Forty seeded random layer shapes (token count, widths, expert count, top-k, dtype, renormalisation)
     against the oracle: every plan boundary gets neighbours on both sides sooner or later."""
