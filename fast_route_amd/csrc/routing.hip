@@ -8,8 +8,9 @@
 // 64 pairs at a time and ranks the pairs of one expert among themselves with
 // wavefront ballots, so flat order survives inside each expert: the result is
 // the stable sort.  Small inputs run all three phases in one workgroup with the
-// tables in LDS; large ones use three launches (count, per-expert segment scan,
-// scatter + block table) and a global table.
+// tables in LDS; large ones use a global table and two launches (count + sums per count
+// workgroup, scatter + block table) or, with many experts, three (count, per-expert
+// segment scan, scatter + block table).
 #include "gating_core.h"
 
 namespace fr {
@@ -62,25 +63,48 @@ __device__ __forceinline__ void segment_histogram(const IdT* __restrict__ ids, i
 
 // Walk [lo, hi) in flat order; cnt[e] holds the next free slot of expert e for
 // this wavefront and is advanced as pairs are placed.
+constexpr int kScatterPF = 4;  // rounds of 64 pairs whose ids are fetched together: the rounds themselves depend on
+                               // one another through cnt[], their loads need not wait for that chain
+template <typename IdT>
+__device__ __forceinline__ void segment_ids(const IdT* __restrict__ ids, int64_t base0, int64_t hi, int lane, int (&ev)[kScatterPF]) {
+#pragma unroll
+  for (int r = 0; r < kScatterPF; ++r) {
+    const int64_t p = base0 + r * kWave + lane;
+    ev[r] = (p < hi) ? static_cast<int>(ids[p]) : -1;
+  }
+}
+// `first`: the ids of the first kScatterPF rounds, fetched by the caller ahead of time (segment_ids), or nullptr
 template <typename IdT>
 __device__ __forceinline__ void segment_scatter(const IdT* __restrict__ ids, int64_t lo, int64_t hi,
                                                 int E, int nbits, int lane, volatile int* cnt,
-                                                int32_t* __restrict__ sorted) {
+                                                int32_t* __restrict__ sorted, const int* first = nullptr) {
   const unsigned long long below = (1ull << lane) - 1ull;
-  for (int64_t base = lo; base < hi; base += kWave) {
-    const int64_t p = base + lane;
-    int e = (p < hi) ? static_cast<int>(ids[p]) : 0;
-    const bool valid = (p < hi) && e >= 0 && e < E;
-    if (!valid) e = 0;
-    const unsigned long long same = same_expert_lanes(e, valid, nbits);
-    if (valid) {
-      const int rank = __popcll(same & below);
-      const int total = __popcll(same);
-      const int old = cnt[e];
-      sorted[old + rank] = static_cast<int32_t>(p);
-      if (rank == total - 1) cnt[e] = old + total;
+  for (int64_t base0 = lo; base0 < hi; base0 += kScatterPF * kWave) {
+    int ev[kScatterPF];
+    if (first != nullptr && base0 == lo) {
+#pragma unroll
+      for (int r = 0; r < kScatterPF; ++r) ev[r] = first[r];
+    } else {
+      segment_ids(ids, base0, hi, lane, ev);
     }
-    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < kScatterPF; ++r) {
+      const int64_t base = base0 + r * kWave;
+      if (base >= hi) break;
+      const int64_t p = base + lane;
+      int e = ev[r];
+      const bool valid = (p < hi) && e >= 0 && e < E;
+      if (!valid) e = 0;
+      const unsigned long long same = same_expert_lanes(e, valid, nbits);
+      if (valid) {
+        const int rank = __popcll(same & below);
+        const int total = __popcll(same);
+        const int old = cnt[e];
+        sorted[old + rank] = static_cast<int32_t>(p);
+        if (rank == total - 1) cnt[e] = old + total;
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
   }
 }
 
@@ -282,6 +306,91 @@ __global__ __launch_bounds__(kSegThreads) void align_scatter_kernel(
   segment_scatter(ids, lo, hi, E, bits_for(E), lane, mine, sorted);
 }
 
+// ---------------------------------------------------------------- large path, two launches
+// The per-expert scan over segments costs a launch of its own only because every scatter workgroup needs
+// (a) each expert's total and (b) the pairs of each expert in the segments before its own.  Here a count
+// workgroup covers 16 segments, leaves each segment's offset INSIDE the workgroup in counts[e][seg] and the
+// workgroup's sums in wgcnt[b][e]; a scatter workgroup then gets (a) and (b) from one pass over the NB x E
+// workgroup sums (6144 values for 64 experts and 393 216 pairs: six loads per thread, summed with integer
+// LDS atomics, so the order does not matter).  Used while NB x E stays small.
+constexpr int kSeg2Threads = 1024;
+constexpr int kSeg2Waves = kSeg2Threads / kWave;
+constexpr int64_t kTwoLevelMaxEntries = 16384;
+
+template <typename IdT>
+__global__ __launch_bounds__(kSeg2Threads) void align_count2_kernel(
+    const IdT* __restrict__ ids, int64_t n, int E, int seg_len, int S, int* __restrict__ counts,
+    int* __restrict__ wgcnt) {
+  extern __shared__ int hist[];  // [kSeg2Waves][E]
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int seg0 = blockIdx.x * kSeg2Waves, seg = seg0 + wave;
+  int* mine = hist + wave * E;
+  for (int e = lane; e < E; e += kWave) mine[e] = 0;
+  __builtin_amdgcn_wave_barrier();
+  if (seg < S) {
+    const int64_t lo = static_cast<int64_t>(seg) * seg_len;
+    const int64_t hi = min64(n, lo + seg_len);
+    segment_histogram(ids, lo, hi, E, lane, mine);
+  }
+  __syncthreads();
+  for (int i = tid; i < E * kSeg2Waves; i += kSeg2Threads) {  // (expert, segment of this workgroup)
+    const int e = i % E, w = i / E;
+    int before = 0;
+    for (int v = 0; v < w; ++v) before += hist[v * E + e];
+    if (seg0 + w < S) counts[static_cast<int64_t>(e) * S + seg0 + w] = before;
+    if (w == kSeg2Waves - 1) wgcnt[static_cast<int64_t>(blockIdx.x) * E + e] = before + hist[w * E + e];
+  }
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(kSeg2Threads) void align_scatter2_kernel(
+    const IdT* __restrict__ ids, int64_t n, int E, int B, int seg_len, int S, int NB, int64_t sorted_len,
+    const int* __restrict__ counts, const int* __restrict__ wgcnt, int32_t* __restrict__ sorted,
+    int32_t* __restrict__ expert_ids, int32_t* __restrict__ npost_out) {
+  extern __shared__ int hist[];  // [kSeg2Waves][E]
+  __shared__ int start[kMaxE + 1];
+  __shared__ int total[kMaxE];
+  __shared__ int before[kMaxE];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wg = blockIdx.x;
+  // this wavefront's segment: its first ids and its offsets inside the workgroup are asked for now, so that
+  // their latency passes together with that of the workgroup sums below
+  const int seg = wg * kSeg2Waves + wave;
+  const int64_t lo = min64(n, static_cast<int64_t>(seg) * seg_len);
+  const int64_t hi = seg < S ? min64(n, lo + seg_len) : lo;
+  int first[kScatterPF];
+  segment_ids(ids, lo, hi, lane, first);
+  const int in_wg0 = (seg < S && lane < E) ? counts[static_cast<int64_t>(lane) * S + seg] : 0;
+  for (int e = tid; e < E; e += kSeg2Threads) total[e] = before[e] = 0;
+  __syncthreads();
+  for (int i = tid; i < E * NB; i += kSeg2Threads) {  // expert e: all pairs, and the pairs in the workgroups before this one
+    const int b = i / E, e = i % E;
+    const int c = wgcnt[i];
+    if (c != 0) {
+      atomicAdd(&total[e], c);
+      if (b < wg) atomicAdd(&before[e], c);
+    }
+  }
+  __syncthreads();
+  if (wave == 0) scan_padded_totals(total, start, E, B, lane);
+  __syncthreads();
+  if (wg < E) {
+    const int e = wg;
+    for (int b = start[e] / B + tid; b < start[e + 1] / B; b += kSeg2Threads) expert_ids[b] = e;
+    for (int s = start[e] + total[e] + tid; s < start[e + 1]; s += kSeg2Threads) sorted[s] = static_cast<int32_t>(n);
+  }
+  if (wg == 0) {
+    for (int64_t s = start[E] + tid; s < sorted_len; s += kSeg2Threads) sorted[s] = static_cast<int32_t>(n);
+    if (tid == 0) npost_out[0] = start[E];
+  }
+  if (seg >= S) return;
+  int* mine = hist + wave * E;
+  if (lane < E) mine[lane] = start[lane] + before[lane] + in_wg0;
+  for (int e = lane + kWave; e < E; e += kWave) mine[e] = start[e] + before[e] + counts[static_cast<int64_t>(e) * S + seg];
+  __builtin_amdgcn_wave_barrier();
+  segment_scatter(ids, lo, hi, E, bits_for(E), lane, mine, sorted, first);
+}
+
 bool use_small_path(int64_t n, int E) { return n <= kSmallMaxN && E <= kSmallMaxE; }
 
 int large_seg_len(int64_t n) {
@@ -308,6 +417,15 @@ int run(const void* ids_v, int64_t n, int E, int B, int32_t* sorted, int32_t* ex
   const unsigned blocks = static_cast<unsigned>(ceil_div(S, kSegWaves));
   const unsigned scatter_blocks = blocks > static_cast<unsigned>(E) ? blocks : static_cast<unsigned>(E);
   const size_t lds = sizeof(int) * kSegWaves * E;
+  const int NB = static_cast<int>(ceil_div(S, kSeg2Waves));
+  if (static_cast<int64_t>(E) * NB <= kTwoLevelMaxEntries && E <= 512) {  // count (+ workgroup sums), scatter: two launches
+    const size_t lds2 = sizeof(int) * kSeg2Waves * E;
+    int* wgcnt = counts + static_cast<int64_t>(E) * S;
+    hipLaunchKernelGGL((align_count2_kernel<IdT>), dim3(NB), dim3(kSeg2Threads), lds2, st, ids, n, E, seg_len, S, counts, wgcnt);
+    hipLaunchKernelGGL((align_scatter2_kernel<IdT>), dim3(NB > E ? NB : E), dim3(kSeg2Threads), lds2, st, ids, n, E, B,
+                       seg_len, S, NB, sorted_len, counts, wgcnt, sorted, expert_ids, npost);
+    return check_launch("align kernels");
+  }
   hipLaunchKernelGGL((align_count_kernel<IdT>), dim3(blocks), dim3(kSegThreads), lds, st, ids, n, E,
                      seg_len, S, counts);
   hipLaunchKernelGGL(align_segscan_kernel, dim3(E), dim3(kSegThreads), 0, st, counts, run_start, S);
@@ -347,8 +465,10 @@ void dispatch_route_align(const void* logits, int64_t M, int E, int topk, int re
 
 // Gating and routing arrays in one launch for small batches; false when the shape is
 // outside what one workgroup should do (the caller then runs the two stages separately).
+// (one workgroup gates and sorts 1024 pairs in 10.5 us; from there on the gating kernel spread over the CUs
+// plus the one-workgroup sort are faster: 8.9 us + a launch gap at 1024 pairs, 12.6 against 26.8 us at 4096)
 bool route_align_fits(int64_t M, int E, int topk) {
-  return M >= 1 && use_small_path(M * topk, E) && M * E <= 16384 && topk <= E;
+  return M >= 1 && M * topk <= 1024 && use_small_path(M * topk, E) && M * E <= 16384 && topk <= E;
 }
 int route_align_small(const void* logits, int logits_dtype, int64_t M, int E, int topk, int renorm, int block,
                       float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost,
@@ -370,7 +490,8 @@ extern "C" int64_t fr_moe_align_workspace_bytes(int64_t n, int E) {
   if (n < 0 || E < 1 || E > kMaxE) return -1;
   if (use_small_path(n, E)) return 0;
   const int64_t S = n > 0 ? ceil_div(n, large_seg_len(n)) : 1;
-  return static_cast<int64_t>(sizeof(int)) * (static_cast<int64_t>(E) * S + E);
+  // [E][S] counts, then E totals (three launches) or [E][ceil(S / 4)] workgroup sums (two launches)
+  return static_cast<int64_t>(sizeof(int)) * (static_cast<int64_t>(E) * S + static_cast<int64_t>(E) * (ceil_div(S, kSegWaves) + 1));
 }
 
 extern "C" int fr_moe_align(const void* topk_ids, int ids_dtype, int64_t n, int E, int block,
