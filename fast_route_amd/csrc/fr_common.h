@@ -27,8 +27,10 @@ const fr_moe_tunables& tunables();
 
 // gating + routing arrays in one launch (small batches); see routing.hip
 bool route_align_fits(int64_t M, int E, int topk);
+// qx (optional): bf16 token rows [M, qK] quantised per row to e4m3 (qq, qscale) by further workgroups of the launch
 int route_align_small(const void* logits, int logits_dtype, int64_t M, int E, int topk, int renorm, int block,
-                      float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, hipStream_t st);
+                      float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost,
+                      const void* qx, int64_t qK, void* qq, float* qscale, hipStream_t st);
 
 #define FR_REQUIRE(cond, code, ...) \
   do {                              \

@@ -173,15 +173,19 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
 namespace fr {
 namespace {
 // top-k gating of the logits and the routing arrays of the result: one launch for small
-// batches, gating then align otherwise
+// batches, gating then align otherwise.  qx (fp8 layer): the bf16 token rows [M, H], quantised per row into
+// c.xq / c.x_scale - by the same launch for small batches, by one of its own otherwise.
 int route_and_align(const void* logits, int logits_dtype, int64_t M, int E, int topk, int renormalize, int block,
-                    const Carve& c, void* stream) {
+                    const Carve& c, const void* qx, int64_t H, void* stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
   if (route_align_fits(M, E, topk))
     return route_align_small(logits, logits_dtype, M, E, topk, renormalize, block, c.topk_w, c.topk_ids, c.sorted,
-                             c.expert_ids, c.npost, static_cast<hipStream_t>(stream));
+                             c.expert_ids, c.npost, qx, H, c.xq, c.x_scale, st);
   int rc = fr_gating_topk(logits, logits_dtype, M, E, E, topk, renormalize, c.topk_w, c.topk_ids, stream);
   if (rc != FR_OK) return rc;
-  return fr_moe_align(c.topk_ids, FR_I32, M * topk, E, block, c.sorted, c.expert_ids, c.npost, c.align_ws, c.align_ws_bytes, stream);
+  rc = fr_moe_align(c.topk_ids, FR_I32, M * topk, E, block, c.sorted, c.expert_ids, c.npost, c.align_ws, c.align_ws_bytes, stream);
+  if (rc != FR_OK || !qx) return rc;
+  return quant_rows(qx, FR_BF16, M, nullptr, H, H, c.xq, c.x_scale, st);
 }
 }  // namespace
 }  // namespace fr
@@ -215,7 +219,7 @@ extern "C" int fr_fused_moe(const void* x, const void* w1, const void* w2, const
   FR_REQUIRE(workspace && workspace_bytes >= p.workspace_bytes, FR_E_WORKSPACE, "fr_fused_moe: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)p.workspace_bytes);
   FR_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FR_E_ALIGN, "fr_fused_moe: workspace must be 256-byte aligned");
   Carve c = carve(workspace, M, H, F, E, topk, dtype, p);
-  rc = route_and_align(logits, logits_dtype, M, E, topk, renormalize, p.block, c, stream);
+  rc = route_and_align(logits, logits_dtype, M, E, topk, renormalize, p.block, c, nullptr, H, stream);
   if (rc != FR_OK) return rc;
   rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, c.tail, stream);
   if (rc != FR_OK) return rc;
@@ -236,9 +240,7 @@ extern "C" int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, con
   FR_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FR_E_ALIGN, "fr_fused_moe_fp8: workspace must be 256-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
   Carve c = carve(workspace, M, H, F, E, topk, FR_FP8_E4M3, p);
-  rc = route_and_align(logits, logits_dtype, M, E, topk, renormalize, p.block, c, stream);
-  if (rc != FR_OK) return rc;
-  rc = quant_rows(x, x_dtype, M, nullptr, H, H, c.xq, c.x_scale, st);
+  rc = route_and_align(logits, logits_dtype, M, E, topk, renormalize, p.block, c, x, H, stream);
   if (rc != FR_OK) return rc;
   rc = fr_moe_gateup_silu_fp8(c.xq, c.x_scale, w1q, w1_scale, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, c.act, stream);
   if (rc != FR_OK) return rc;

@@ -12,6 +12,7 @@
 // workgroup, scatter + block table) or, with many experts, three (count, per-expert
 // segment scan, scatter + block table).
 #include "gating_core.h"
+#include "quant_core.h"
 
 namespace fr {
 namespace {
@@ -180,6 +181,14 @@ __global__ __launch_bounds__(kSmallThreads) void align_small_kernel(
   segment_scatter(ids, lo, hi, E, bits_for(E), lane, &table[wave * E], sorted);
 }
 
+// bf16 token rows [M, K] to quantise to e4m3 alongside (x == nullptr: none)
+struct RowQuant {
+  const bf16_t* x;
+  unsigned char* q;
+  float* scale;
+  int K;
+};
+
 // Small batches, whole routing in one launch: the workgroup first gates every token
 // (a group of G lanes per token, 1024/G tokens per pass; weights and ids go to their
 // global arrays), then sorts the ids it has just written exactly as above.
@@ -187,11 +196,16 @@ template <typename T, int G, int VPL>
 __global__ __launch_bounds__(kSmallThreads) void route_align_small_kernel(
     const T* __restrict__ logits, int64_t M, int E, int topk, int renorm, int B, int seg_len, int64_t sorted_len,
     float* __restrict__ w_out, int32_t* __restrict__ ids_out, int32_t* __restrict__ sorted,
-    int32_t* __restrict__ expert_ids, int32_t* __restrict__ npost_out) {
+    int32_t* __restrict__ expert_ids, int32_t* __restrict__ npost_out, RowQuant rq) {
   __shared__ int table[kSmallWaves * kSmallMaxE];
   __shared__ int total[kSmallMaxE];
   __shared__ int start[kSmallMaxE + 1];
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  if (blockIdx.x > 0) {  // the fp8 layer's token rows are quantised by further workgroups of the same launch
+    const int64_t row = static_cast<int64_t>(blockIdx.x - 1) * kSmallWaves + wave;
+    if (row < M) quant_row(rq.x + row * rq.K, rq.K, rq.q + row * rq.K, rq.scale + row, lane);
+    return;
+  }
   for (int i = tid; i < kSmallWaves * E; i += kSmallThreads) table[i] = 0;
   constexpr int kPerPass = kSmallThreads / G;
   for (int64_t base = 0; base < M; base += kPerPass) {  // uniform trip count: every lane joins the cross-lane ops
@@ -436,19 +450,21 @@ int run(const void* ids_v, int64_t n, int E, int B, int32_t* sorted, int32_t* ex
 
 template <typename T, int G, int VPL>
 void launch_route_align(const void* logits, int64_t M, int E, int topk, int renorm, int B, int64_t sorted_len,
-                        float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, hipStream_t st) {
+                        float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, RowQuant rq,
+                        hipStream_t st) {
   int seg_len = static_cast<int>(round_up(ceil_div(M * topk, kSmallWaves), kWave));
   if (seg_len == 0) seg_len = kWave;
-  hipLaunchKernelGGL((route_align_small_kernel<T, G, VPL>), dim3(1), dim3(kSmallThreads), 0, st,
+  const unsigned grid = 1 + (rq.x ? static_cast<unsigned>(ceil_div(M, kSmallWaves)) : 0u);
+  hipLaunchKernelGGL((route_align_small_kernel<T, G, VPL>), dim3(grid), dim3(kSmallThreads), 0, st,
                      static_cast<const T*>(logits), M, E, topk, renorm, B, seg_len, sorted_len, w, ids, sorted,
-                     expert_ids, npost);
+                     expert_ids, npost, rq);
 }
 
 template <typename T>
 void dispatch_route_align(const void* logits, int64_t M, int E, int topk, int renorm, int B, int64_t sorted_len,
-                          float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost,
+                          float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, RowQuant rq,
                           hipStream_t st) {
-#define FR_RA(G, VPL) launch_route_align<T, G, VPL>(logits, M, E, topk, renorm, B, sorted_len, w, ids, sorted, expert_ids, npost, st)
+#define FR_RA(G, VPL) launch_route_align<T, G, VPL>(logits, M, E, topk, renorm, B, sorted_len, w, ids, sorted, expert_ids, npost, rq, st)
   if (E <= 1) FR_RA(1, 1);
   else if (E <= 2) FR_RA(2, 1);
   else if (E <= 4) FR_RA(4, 1);
@@ -472,12 +488,13 @@ bool route_align_fits(int64_t M, int E, int topk) {
 }
 int route_align_small(const void* logits, int logits_dtype, int64_t M, int E, int topk, int renorm, int block,
                       float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost,
-                      hipStream_t st) {
+                      const void* qx, int64_t qK, void* qq, float* qscale, hipStream_t st) {
   const int64_t sorted_len = M * topk + int64_t(E) * (block - 1);
+  const RowQuant rq = {static_cast<const bf16_t*>(qx), static_cast<unsigned char*>(qq), qscale, static_cast<int>(qK)};
   switch (logits_dtype) {
-    case FR_F32: dispatch_route_align<float>(logits, M, E, topk, renorm, block, sorted_len, w, ids, sorted, expert_ids, npost, st); break;
-    case FR_F16: dispatch_route_align<f16_t>(logits, M, E, topk, renorm, block, sorted_len, w, ids, sorted, expert_ids, npost, st); break;
-    case FR_BF16: dispatch_route_align<bf16_t>(logits, M, E, topk, renorm, block, sorted_len, w, ids, sorted, expert_ids, npost, st); break;
+    case FR_F32: dispatch_route_align<float>(logits, M, E, topk, renorm, block, sorted_len, w, ids, sorted, expert_ids, npost, rq, st); break;
+    case FR_F16: dispatch_route_align<f16_t>(logits, M, E, topk, renorm, block, sorted_len, w, ids, sorted, expert_ids, npost, rq, st); break;
+    case FR_BF16: dispatch_route_align<bf16_t>(logits, M, E, topk, renorm, block, sorted_len, w, ids, sorted, expert_ids, npost, rq, st); break;
     default: return fail(FR_E_DTYPE, "route_align_small: logits dtype %d not in {f32, f16, bf16}", logits_dtype);
   }
   return check_launch("route_align_small_kernel");

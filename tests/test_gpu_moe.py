@@ -612,6 +612,44 @@ def test_tunables_and_prepare(native):
     assert torch.equal(fused_moe(xd, w1d, w2d, ld, 2, True), base)
 
 
+@pytest.mark.parametrize("block", [128, 256])
+@pytest.mark.parametrize("kind", ["bf16", "fp8"])
+def test_persistent_tiles_alternating_half_empty_and_full_blocks(native, block, kind):
+    """The persistent 128- and 256-row kernels let the wavefronts of a block's upper half skip their fragment
+    reads and MFMAs when that half holds only padding, and pick the fragments up again when their next block
+    has rows.  64 experts with one routing block each, a seeded mix of full blocks and blocks filled to less
+    than half, 8 feature tiles per block: every workgroup walks several units and meets both transitions."""
+    import fast_route_amd as fr
+    from fast_route_amd import fused_experts, fused_moe_fp8, prepare_weights_fp8
+    E, H, Fd = 64, 512, 1024
+    rng = np.random.default_rng(block)
+    counts = np.where(rng.random(E) < 0.5, block, rng.integers(1, block // 2 + 1, E))
+    ids = torch.from_numpy(np.repeat(np.arange(E), counts)).int()
+    ids = ids[torch.from_numpy(rng.permutation(ids.numel()))].view(-1, 1)
+    M = ids.shape[0]
+    _say(f"persistent half/full blocks block={block} {kind} M={M}")
+    x, _, w1, w2 = _inputs(M, H, Fd, E, 31 + block, torch.bfloat16)
+    try:
+        with fr.tunables(block=block):
+            if kind == "bf16":
+                wts = torch.rand(M, 1) + 0.5
+                out = fused_experts(x.cuda(), w1.cuda(), w2.cuda(), wts.cuda(), ids.cuda())
+                torch.cuda.synchronize()
+                _assert_close(out, oracle.moe_experts(x, w1, w2, wts, ids), torch.bfloat16, "half/full blocks")
+            else:
+                logits = torch.full((M, E), -20.0)
+                logits[torch.arange(M), ids.view(-1).long()] = 20.0
+                w1q, w1s, w2q, w2s = prepare_weights_fp8(w1.cuda(), w2.cuda())
+                out = fused_moe_fp8(x.cuda(), w1q, w1s, w2q, w2s, logits.cuda(), 1, True)
+                torch.cuda.synchronize()
+                ref, _ = oracle.fused_moe_fp8(x, w1, w2, logits, 1, True)
+                o = out.float().cpu()
+                assert torch.isfinite(o).all()
+                assert (o - ref).norm() / ref.norm() <= 1e-2 and (o - ref).abs().max() <= 2.0 ** -5 * ref.abs().max()
+    finally:
+        fr.reset_tunables()
+
+
 def test_random_shapes_against_oracle(native):
     """Forty seeded random layer shapes (token count, widths, expert count, top-k, dtype, renormalisation)
     against the oracle: every plan boundary gets neighbours on both sides sooner or later."""
