@@ -328,27 +328,20 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
   // ---- per-lane fragment rows ---------------------------------------------
   const int frow = lane % C::TILE;  // row inside an MFMA tile
   const int kgrp = lane / C::TILE;  // which K group of the MFMA this lane feeds
-  int xoff[C::IT], woff[C::JF];     // chunk offset of the lane's row
-  int xkey[C::IT], wkey[C::JF];     // swizzle key of that row
-#pragma unroll
-  for (int i = 0; i < C::IT; ++i) {
-    const int r = wt * C::TT + i * C::TILE + frow;
-    xoff[i] = r * CPR;
-    xkey[i] = swizzle<CPR>(r, 0);
-  }
-#pragma unroll
-  for (int j = 0; j < C::JF; ++j) {
-    int base;
-    if constexpr (EPI == EPI_SILU) {
-      constexpr int HJ = C::JF / 2;  // first half of the wave's tiles: gate, second: up
-      base = (j < HJ) ? wf * (C::TF / 2) + j * C::TILE : BF / 2 + wf * (C::TF / 2) + (j - HJ) * C::TILE;
-    } else {
-      base = wf * C::TF + j * C::TILE;
-    }
-    const int r = base + frow;
-    woff[j] = WBASE + r * CPR;
-    wkey[j] = swizzle<CPR>(r, 0);
-  }
+  // All fragment rows of a lane lie a multiple of 16 rows apart, which leaves the swizzle key unchanged: one
+  // offset and one key per operand, the fragments at compile-time distances from them (immediate offsets of
+  // the LDS reads).
+  static_assert(C::TILE % 16 == 0 && (BF / 2) % 16 == 0 && C::TF % 16 == 0 && C::TT % 16 == 0, "fragment rows 16 apart");
+  constexpr int HJ_ = C::JF / 2;  // EPI_SILU: first half of the wave's tiles gate rows, second half the matching up rows
+  auto wcol = [](int wf_, int j) constexpr -> int {
+    if (EPI == EPI_SILU) return (j < HJ_) ? wf_ * (C::TF / 2) + j * C::TILE : BF / 2 + wf_ * (C::TF / 2) + (j - HJ_) * C::TILE;
+    return wf_ * C::TF + j * C::TILE;
+  };
+  const int xrow0 = wt * C::TT + frow, wrow0 = wcol(wf, 0) + frow;
+  const int xoff0 = xrow0 * CPR, xkey0 = swizzle<CPR>(xrow0, 0);
+  const int woff0 = WBASE + wrow0 * CPR, wkey0 = swizzle<CPR>(wrow0, 0);
+#define FR_XD(i_) ((i_) * C::TILE * CPR)
+#define FR_WD(j_) ((wcol(0, (j_)) - wcol(0, 0)) * CPR)
 
   acc_t acc[C::JF][C::IT];
 #pragma unroll
@@ -366,10 +359,10 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     const u32x4* wtl = lds + (ws_) * C::WCH;                                            \
     _Pragma("unroll") for (int c = 0; c < FC; ++c) {                                    \
       const int kc = ((ks_) * C::KGROUPS + kgrp) * FC + c;                              \
-      _Pragma("unroll") for (int i = 0; i < C::IT; ++i)                                 \
-        xf[fb_][i][c] = xt[xoff[i] + (kc ^ xkey[i])];                                   \
-      _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                                 \
-        wfr[fb_][j][c] = wtl[woff[j] + (kc ^ wkey[j])];                                 \
+      const u32x4* xp_ = xt + xoff0 + (kc ^ xkey0);                                     \
+      const u32x4* wp_ = wtl + woff0 + (kc ^ wkey0);                                    \
+      _Pragma("unroll") for (int i = 0; i < C::IT; ++i) xf[fb_][i][c] = xp_[FR_XD(i)];  \
+      _Pragma("unroll") for (int j = 0; j < C::JF; ++j) wfr[fb_][j][c] = wp_[FR_WD(j)]; \
     }                                                                                   \
   }
 #define FR_MMA(fb_, j0_, j1_)                                                           \
@@ -615,6 +608,8 @@ _Pragma("unroll") \
   }
 #undef FR_READ_FRAGS
 #undef FR_MMA
+#undef FR_XD
+#undef FR_WD
 
   gemm_epilogue<T, C, EPI>(a, acc, pid_t, pid_f, expert, split, wt, wf, frow, kgrp);
 }

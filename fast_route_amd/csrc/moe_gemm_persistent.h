@@ -150,7 +150,10 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
   constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, IW = C::IW, NLI = (XI + WI) * IW;
   constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
-  constexpr bool SINGLE = E::SCALED;   // one fragment buffer for fp8 (8-register fragments), two otherwise
+#ifndef FR_SINGLE_FRAG
+#define FR_SINGLE_FRAG false
+#endif
+  constexpr bool SINGLE = E::SCALED || FR_SINGLE_FRAG;   // one fragment buffer for fp8 (8-register fragments), two otherwise
   static_assert(S >= 2 && C::SPREAD <= 1, "persistent form: ring of at least two slots, refill in one group");
   static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
   static_assert((S - 1) * NLI <= 63, "vmcnt budget");
@@ -220,20 +223,15 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 
   // ---- per-lane fragment rows ---------------------------------------------------
   const int frow = lane % C::TILE, kgrp = lane / C::TILE;
-  int xoff[C::IT], woff[C::JF], xkey[C::IT], wkey[C::JF];
-#pragma unroll
-  for (int i = 0; i < C::IT; ++i) {
-    const int r = wt * C::TT + i * C::TILE + frow;
-    xoff[i] = r * CPR;
-    xkey[i] = swizzle<CPR>(r, 0);
-  }
-#pragma unroll
-  for (int j = 0; j < C::JF; ++j) {
-    const int base = acc_tile_col<C, EPI>(wf, j);
-    const int r = base + frow;
-    woff[j] = WBASE + r * CPR;
-    wkey[j] = swizzle<CPR>(r, 0);
-  }
+  // All fragment rows of a lane lie a multiple of 16 rows apart, which leaves the swizzle key unchanged: one
+  // offset and one key per operand, the fragments at compile-time distances from them (immediate offsets of
+  // the LDS reads).
+  static_assert(C::TILE % 16 == 0 && (BF / 2) % 16 == 0 && C::TF % 16 == 0 && C::TT % 16 == 0, "fragment rows 16 apart");
+  const int xrow0 = wt * C::TT + frow, wrow0 = acc_tile_col<C, EPI>(wf, 0) + frow;
+  const int xoff0 = xrow0 * CPR, xkey0 = swizzle<CPR>(xrow0, 0);
+  const int woff0 = WBASE + wrow0 * CPR, wkey0 = swizzle<CPR>(wrow0, 0);
+#define FR_XD(i_) ((i_) * C::TILE * CPR)
+#define FR_WD(j_) ((acc_tile_col<C, EPI>(0, (j_)) - acc_tile_col<C, EPI>(0, 0)) * CPR)
   acc_t acc[C::JF][C::IT];
   u32x4 xf[2][C::IT][FC], wfr[2][C::JF][FC];
 
@@ -287,10 +285,10 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     const u32x4* wtl = lds + (sl_) * C::WCH;                                            \
     _Pragma("unroll") for (int c = 0; c < FC; ++c) {                                    \
       const int kc = ((ks_) * C::KGROUPS + kgrp) * FC + c;                              \
-      _Pragma("unroll") for (int i = 0; i < C::IT; ++i)                                 \
-        xf[fb_][i][c] = xt[xoff[i] + (kc ^ xkey[i])];                                   \
-      _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                                 \
-        wfr[fb_][j][c] = wtl[woff[j] + (kc ^ wkey[j])];                                 \
+      const u32x4* xp_ = xt + xoff0 + (kc ^ xkey0);                                     \
+      const u32x4* wp_ = wtl + woff0 + (kc ^ wkey0);                                    \
+      _Pragma("unroll") for (int i = 0; i < C::IT; ++i) xf[fb_][i][c] = xp_[FR_XD(i)];  \
+      _Pragma("unroll") for (int j = 0; j < C::JF; ++j) wfr[fb_][j][c] = wp_[FR_WD(j)]; \
     }                                                                                   \
   }
   // fragment i_ of the token operand / j_ of the weight operand alone, into buffer 0
@@ -299,7 +297,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     const u32x4* xt = lds + (sl_) * C::XCH;                                             \
     _Pragma("unroll") for (int c = 0; c < FC; ++c) {                                    \
       const int kc = ((ks_) * C::KGROUPS + kgrp) * FC + c;                              \
-      xf[0][i_][c] = xt[xoff[i_] + (kc ^ xkey[i_])];                                    \
+      xf[0][i_][c] = xt[xoff0 + (kc ^ xkey0) + FR_XD(i_)];                              \
     }                                                                                   \
   }
 #define FR_READ_W1(sl_, ks_, j_)                                                        \
@@ -307,7 +305,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     const u32x4* wtl = lds + (sl_) * C::WCH;                                            \
     _Pragma("unroll") for (int c = 0; c < FC; ++c) {                                    \
       const int kc = ((ks_) * C::KGROUPS + kgrp) * FC + c;                              \
-      wfr[0][j_][c] = wtl[woff[j_] + (kc ^ wkey[j_])];                                  \
+      wfr[0][j_][c] = wtl[woff0 + (kc ^ wkey0) + FR_WD(j_)];                            \
     }                                                                                   \
   }
   // One K-step: NM MFMAs, weight tile j outer, token tile i inner.  HAVE_NEXT: the fragments of K-step
@@ -441,6 +439,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #undef FR_KTILE
 #undef FR_KSTEP
 #undef FR_READ_W1
+#undef FR_XD
+#undef FR_WD
 #undef FR_READ_X1
 #undef FR_READ_FRAGS
 #undef FR_ISSUE_ONE
