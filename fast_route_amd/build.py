@@ -40,15 +40,18 @@ def _run(cmd):
 
 
 def build(verbose: bool = False) -> str:
-    """Compiles every source and links the shared library; returns its path."""
+    """Compiles every source and links the shared library; returns its path.
+    FR_HIPCC_FLAGS in the environment adds compiler flags (the measurement switches of
+    csrc/moe_gemm_persistent.h, e.g. FR_HIPCC_FLAGS="-DFR_ABL_NOLOAD")."""
     hipcc = _hipcc()
+    extra = os.environ.get("FR_HIPCC_FLAGS", "").split()
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
 
     def one(pair):
         src, obj = pair
-        return _run([hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+        return _run([hipcc, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj])
 
     with ThreadPoolExecutor(max_workers=min(os.cpu_count() or 8, 16, len(SOURCES))) as pool:
         for out in pool.map(one, zip(SOURCES, objs)):

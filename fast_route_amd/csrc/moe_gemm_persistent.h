@@ -150,10 +150,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
   constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, IW = C::IW, NLI = (XI + WI) * IW;
   constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
-#ifndef FR_SINGLE_FRAG
-#define FR_SINGLE_FRAG false
-#endif
-  constexpr bool SINGLE = E::SCALED || FR_SINGLE_FRAG;   // one fragment buffer for fp8 (8-register fragments), two otherwise
+  constexpr bool SINGLE = E::SCALED;   // one fragment buffer for fp8 (8-register fragments), two otherwise
   static_assert(S >= 2 && C::SPREAD <= 1, "persistent form: ring of at least two slots, refill in one group");
   static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
   static_assert((S - 1) * NLI <= 63, "vmcnt budget");
@@ -265,8 +262,13 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   FR_UNIT(0, pid_t, pid_f, expert, kb, kn, tu)
   FR_MAKE_SET(pid_t, pid_f, expert, kb, a.sorted[pid_t * BT + rr], xsrcA, wsrcA, xrsA, wrsA)
 
+  // Measurement switches (compile time; results are WRONG with any of them, only timings mean something):
+  //   FR_ABL_NOLOAD  the ring is filled once and never refilled: MFMAs + fragment reads + barriers on real data
+  //   FR_ABL_NOLDS   (with NOLOAD) fragments are read once and stay in registers: MFMAs + barriers
+  //   FR_ABL_NOBAR   no barrier between K tiles
+  // They split a launch's time into its MFMA floor, the cost of the LDS fragment reads and the cost of the tile loads.
   // load q_ of an issuing wavefront (weight-tile loads first) of K tile tile_ into ring slot slot_
-#define FR_ISSUE_ONE(SET, tile_, slot_, q_)                                                                 \
+#define FR_ISSUE_REAL(SET, tile_, slot_, q_)                                                                \
   {                                                                                                         \
     const int vwi_ = wave_u + ((q_) % IW) * (NW / IW);                                                      \
     if ((q_) < WI * IW) {                                                                                   \
@@ -279,7 +281,12 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
           16, xsrc##SET[(q_) < WI * IW ? 0 : (q_) - WI * IW], (tile_) * C::BKB, 0, 0);                      \
     }                                                                                                       \
   }
-#define FR_READ_FRAGS(sl_, ks_, fb_)                                                    \
+#ifdef FR_ABL_NOLOAD
+#define FR_ISSUE_ONE(SET, tile_, slot_, q_) {}
+#else
+#define FR_ISSUE_ONE(SET, tile_, slot_, q_) FR_ISSUE_REAL(SET, tile_, slot_, q_)
+#endif
+#define FR_READ_FRAGS_REAL(sl_, ks_, fb_)                                               \
   {                                                                                     \
     const u32x4* xt = lds + (sl_) * C::XCH;                                             \
     const u32x4* wtl = lds + (sl_) * C::WCH;                                            \
@@ -291,6 +298,18 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
       _Pragma("unroll") for (int j = 0; j < C::JF; ++j) wfr[fb_][j][c] = wp_[FR_WD(j)]; \
     }                                                                                   \
   }
+#ifdef FR_ABL_NOLDS
+#define FR_READ_FRAGS(sl_, ks_, fb_) {}
+#define FR_ABL_INIT1 FR_READ_FRAGS_REAL(0, 1, 1);
+#else
+#define FR_READ_FRAGS(sl_, ks_, fb_) FR_READ_FRAGS_REAL(sl_, ks_, fb_)
+#define FR_ABL_INIT1
+#endif
+#ifdef FR_ABL_NOBAR
+#define FR_KT_BARRIER
+#else
+#define FR_KT_BARRIER __builtin_amdgcn_s_barrier();
+#endif
   // fragment i_ of the token operand / j_ of the weight operand alone, into buffer 0
 #define FR_READ_X1(sl_, ks_, i_)                                                        \
   {                                                                                     \
@@ -356,7 +375,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
         FR_KSTEP(ks & 1, false, 0, 0, false, A, 0, 0);                                         \
       } else {                                                                                 \
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(VMC) : "memory");                  \
-        __builtin_amdgcn_s_barrier();                                                          \
+        FR_KT_BARRIER                                                                          \
         FR_KSTEP(ks & 1, true, sn, 0, (ISS_) && (REFILL), SET, rtile_, sl);                    \
       }                                                                                        \
     }                                                                                          \
@@ -412,10 +431,11 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #define FR_FILL(ISS_)                                                                                      \
   {                                                                                                        \
     _Pragma("unroll") for (int t = 0; t < S; ++t)                                                          \
-      if (ISS_) { _Pragma("unroll") for (int q = 0; q < NLI; ++q) FR_ISSUE_ONE(A, t, t, q); }               \
+      if (ISS_) { _Pragma("unroll") for (int q = 0; q < NLI; ++q) FR_ISSUE_REAL(A, t, t, q); }              \
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((S - 1) * NLI) : "memory");                                   \
     __builtin_amdgcn_s_barrier();                                                                          \
-    FR_READ_FRAGS(0, 0, 0);                                                                                \
+    FR_READ_FRAGS_REAL(0, 0, 0);                                                                           \
+    FR_ABL_INIT1                                                                                           \
   }
   // Whole pipeline for an issuing (ISS_ = true) or a non-issuing wavefront.
 #define FR_PERSIST(ISS_)                                                                                   \
@@ -444,6 +464,10 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #undef FR_READ_X1
 #undef FR_READ_FRAGS
 #undef FR_ISSUE_ONE
+#undef FR_ISSUE_REAL
+#undef FR_READ_FRAGS_REAL
+#undef FR_ABL_INIT1
+#undef FR_KT_BARRIER
 #undef FR_MAKE_SET
 #undef FR_SLOT_ROW
 #undef FR_UNIT

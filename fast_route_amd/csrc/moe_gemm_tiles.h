@@ -18,11 +18,8 @@ namespace fr {
 //                   weight streaming at HBM rate.  The gate/up GEMM (short weight rows
 //                   of H elements, many of them) streams faster with 512-byte row
 //                   segments: T32L / T16L, used when H allows.
-#ifndef FR_T256_CFG
-#define FR_T256_CFG 256, 256, 128, 2, 4, 32, 1, 2, 0, 2
-#endif
 template <typename T> struct Tiles {  // bf16 / fp16
-  typedef Cfg<FR_T256_CFG> T256;
+  typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;  // persistent form; one wavefront per SIMD issues the loads (2-4 % over each its own)
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 3, 3> T64;    // 3-slot ring like the 128-row tile (5 % over the register-staged form)
