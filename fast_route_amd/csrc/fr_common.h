@@ -32,6 +32,12 @@ int route_align_small(const void* logits, int logits_dtype, int64_t M, int E, in
                       float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost,
                       const void* qx, int64_t qK, void* qq, float* qscale, hipStream_t st);
 
+// Gate/up projection of a handful of tokens that does the layer's routing itself (see moe_gemv.h).  Returns
+// FR_OK, an error, or 1 when the shape is not one it takes (nothing launched: route and project separately).
+int gateup_rows_routed(const void* x, const void* w1, const void* logits, int logits_dtype, int64_t M, int64_t H,
+                       int64_t F, int E, int topk, int renorm, int block, int dtype, void* act, float* topk_w,
+                       int32_t* topk_ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, hipStream_t st);
+
 #define FR_REQUIRE(cond, code, ...) \
   do {                              \
     if (!(cond)) return ::fr::fail((code), __VA_ARGS__); \

@@ -219,10 +219,16 @@ extern "C" int fr_fused_moe(const void* x, const void* w1, const void* w2, const
   FR_REQUIRE(workspace && workspace_bytes >= p.workspace_bytes, FR_E_WORKSPACE, "fr_fused_moe: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)p.workspace_bytes);
   FR_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FR_E_ALIGN, "fr_fused_moe: workspace must be 256-byte aligned");
   Carve c = carve(workspace, M, H, F, E, topk, dtype, p);
-  rc = route_and_align(logits, logits_dtype, M, E, topk, renormalize, p.block, c, nullptr, H, stream);
-  if (rc != FR_OK) return rc;
-  rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, c.tail, stream);
-  if (rc != FR_OK) return rc;
+  // a handful of tokens: the gate/up launch gates and sorts by itself
+  rc = gateup_rows_routed(x, w1, logits, logits_dtype, M, H, F, E, topk, renormalize, p.block, dtype, c.act, c.topk_w,
+                          c.topk_ids, c.sorted, c.expert_ids, c.npost, static_cast<hipStream_t>(stream));
+  if (rc < 0) return rc;
+  if (rc == 1) {
+    rc = route_and_align(logits, logits_dtype, M, E, topk, renormalize, p.block, c, nullptr, H, stream);
+    if (rc != FR_OK) return rc;
+    rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, c.tail, stream);
+    if (rc != FR_OK) return rc;
+  }
   return fr_moe_down_combine(c.act, w2, c.topk_w, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, p.split_k, dtype, c.partial, out, c.tail, stream);
 }
 

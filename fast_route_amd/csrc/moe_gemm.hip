@@ -131,6 +131,27 @@ int gateup_impl(const void* x, const float* x_scale, const void* w1, const float
   return dispatch_dtype<EPI_SILU>(a, dtype, block, 1, sorted_len / block * block, st);
 }
 
+int gateup_rows_routed(const void* x, const void* w1, const void* logits, int logits_dtype, int64_t M, int64_t H,
+                       int64_t F, int E, int topk, int renorm, int block, int dtype, void* act, float* topk_w,
+                       int32_t* topk_ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, hipStream_t st) {
+  const int64_t n = M * topk, sorted_len = n + int64_t(E) * (block - 1);
+  if ((dtype != FR_BF16 && dtype != FR_F16) || !gateup_rows_fits(M, H, block, sorted_len, 2) ||
+      !gateup_rows_routes(M, E, topk, block) || F % 8 != 0 ||
+      (logits_dtype != FR_F32 && logits_dtype != FR_F16 && logits_dtype != FR_BF16))
+    return 1;
+  FR_REQUIRE(x && w1 && logits && act && topk_w && topk_ids && sorted && expert_ids && npost, FR_E_NULL, "gate/up with routing: null pointer");
+  FR_REQUIRE(aligned16(x) && aligned16(w1) && aligned16(act), FR_E_ALIGN, "gate/up with routing: operands must be 16-byte aligned");
+  GemmArgs a = {};
+  a.X = x; a.ldx = H; a.W = w1; a.w_expert_stride = 2 * F * H; a.ldw = H; a.out = act; a.ldo = F;
+  a.sorted = sorted; a.expert_ids = expert_ids; a.npost = npost;
+  a.w_rows = static_cast<int>(2 * F);
+  a.num_valid = (int)n; a.top_k = topk; a.N = (int)F; a.K = (int)H;
+  a.num_experts = E;
+  const RowsRoute rt = {logits, logits_dtype, E, topk, renorm, topk_w, topk_ids, sorted, expert_ids, npost};
+  if (dtype == FR_BF16) return launch_gateup_rows<bf16_t>(a, block, sorted_len / block * block, st, rt);
+  return launch_gateup_rows<f16_t>(a, block, sorted_len / block * block, st, rt);
+}
+
 int down_impl(const void* act, const float* act_scale, const void* w2, const float* w2_scale,
               const float* topk_weights, const int32_t* sorted, const int32_t* expert_ids, const int32_t* npost,
               int64_t M, int64_t H, int64_t F, int E, int topk, int block, int split_k, int dtype, int out_dtype,

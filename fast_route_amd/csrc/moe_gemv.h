@@ -14,6 +14,7 @@
 // the token rows are in LDS.  Same arguments and output layout as the EPI_SILU
 // tile kernel (act[slot, F]), so the down projection that follows is unchanged.
 #pragma once
+#include "gating_core.h"
 #include "moe_gemm_kernel.h"
 
 namespace fr {
@@ -23,7 +24,7 @@ constexpr int kRowsThreads = 256;  // 4 wavefronts
 constexpr int kRowsMinK = 4096;    // shorter rows: the tile kernel is as fast (measured at 1024 and 2048)
 constexpr int kRowsWaves = 4096;   // wavefronts the feature runs are cut for: 16 on each of 256 CUs
 constexpr int kRowsWaveBytes = 7 * 16384;  // weight bytes a wavefront streams
-constexpr int kRowsLds = 65536;    // token rows in LDS: the default dynamic limit
+constexpr int kRowsLds = 62464;    // token rows in LDS: the default limit of 64 KB less the kernel's static arrays
 
 template <typename T> struct Dot2;
 template <> struct Dot2<bf16_t> {
@@ -49,6 +50,47 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Routing done by the gate/up launch itself (whole layer from router logits, up to kRowsMax tokens): every
+// workgroup gates the tokens and sorts the few pairs for itself in LDS - the same gating core and the same
+// order as the routing kernels - and workgroup (0, 0) also leaves the arrays in global memory for the down
+// projection.  One launch and its gap less in front of a layer that lasts ~110 us.
+struct RowsRoute {
+  const void* logits;   // [M, E] dense, or nullptr: the routing arrays of GemmArgs are read instead
+  int logits_dtype;
+  int E, topk, renorm;
+  float* w_out;         // [M, topk]
+  int32_t* ids_out;     // [M, topk]
+  int32_t* sorted_out;  // first npost entries written
+  int32_t* expert_out;  // first npost / block entries written
+  int32_t* npost_out;
+};
+constexpr int kRowsPairs = 32;                  // pairs at most (kRowsMax tokens x topk <= 8)
+constexpr int kRowsSlots = kRowsPairs * 16;     // slots of the in-LDS routing arrays (blocks of 16)
+
+template <typename LT, int G, int VPL>
+__device__ __forceinline__ void rows_gate_as(const LT* logits, int M, int E, int topk, int renorm, float* w, int32_t* ids) {
+  constexpr int PER = kWave / G;  // tokens per pass of one wavefront
+  const int lane = threadIdx.x & (kWave - 1);
+  for (int base = 0; base < M; base += PER) {
+    const int token = base + lane / G;
+    const bool live = token < M;
+    const LT* row = logits + static_cast<int64_t>(live ? token : 0) * E;
+    gate_token<G, VPL>([&](int e) { return to_float(row[e]); }, live, E, topk, renorm, w + token * topk, ids + token * topk);
+  }
+}
+template <typename LT>
+__device__ __forceinline__ void rows_gate(const LT* logits, int M, int E, int topk, int renorm, float* w, int32_t* ids) {
+  if (E <= 1) rows_gate_as<LT, 1, 1>(logits, M, E, topk, renorm, w, ids);
+  else if (E <= 2) rows_gate_as<LT, 2, 1>(logits, M, E, topk, renorm, w, ids);
+  else if (E <= 4) rows_gate_as<LT, 4, 1>(logits, M, E, topk, renorm, w, ids);
+  else if (E <= 8) rows_gate_as<LT, 8, 1>(logits, M, E, topk, renorm, w, ids);
+  else if (E <= 16) rows_gate_as<LT, 16, 1>(logits, M, E, topk, renorm, w, ids);
+  else if (E <= 32) rows_gate_as<LT, 32, 1>(logits, M, E, topk, renorm, w, ids);
+  else if (E <= 64) rows_gate_as<LT, 64, 1>(logits, M, E, topk, renorm, w, ids);
+  else if (E <= 128) rows_gate_as<LT, 64, 2>(logits, M, E, topk, renorm, w, ids);
+  else rows_gate_as<LT, 64, 4>(logits, M, E, topk, renorm, w, ids);
+}
+
 // CH = 16-byte chunks per lane, row and round: a weight row is `rounds` x CH x 512 elements (CH = 8 for K = 4096
 // and 8192, 5 for 5120, 6 for 6144, 7 for 7168); a lane has 2 * CH loads in flight.
 // grid.x * 4 wavefronts cover the F features in runs of `fpw`; grid.y = routing blocks (upper bound).
@@ -56,18 +98,79 @@ __device__ __forceinline__ float wave_sum(float v) {
 // selects an expert once, so all rows of a block are in its first pass and the later passes find
 // nothing; ids with repeated experts per token still come out right, at one more pass over the weights.
 template <typename T, int CH>
-__global__ void __launch_bounds__(kRowsThreads) gateup_rows_kernel(GemmArgs a, int block, int rows, int fpw) {
+__global__ void __launch_bounds__(kRowsThreads) gateup_rows_kernel(GemmArgs a, int block, int rows, int fpw, RowsRoute rt) {
   extern __shared__ u32x4 xs[];  // rows x K/8 chunks
+  __shared__ float r_w[kRowsPairs];
+  __shared__ int32_t r_ids[kRowsPairs], r_sorted[kRowsSlots], r_expert[kRowsPairs], r_npost;
   const int b = blockIdx.y;
-  if (b * block >= *a.npost) return;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int32_t* sorted = a.sorted;
+  const int32_t* expert_ids = a.expert_ids;
+  int npost;
+  if (rt.logits != nullptr) {
+    // ---- routing in LDS: gating by wavefront 0, then the stable sort of the n <= kRowsPairs pairs ----
+    const int M = a.num_valid / a.top_k, n = a.num_valid;
+    if (wave == 0) {
+      if (rt.logits_dtype == FR_F32) rows_gate(static_cast<const float*>(rt.logits), M, rt.E, rt.topk, rt.renorm, r_w, r_ids);
+      else if (rt.logits_dtype == FR_BF16) rows_gate(static_cast<const bf16_t*>(rt.logits), M, rt.E, rt.topk, rt.renorm, r_w, r_ids);
+      else rows_gate(static_cast<const f16_t*>(rt.logits), M, rt.E, rt.topk, rt.renorm, r_w, r_ids);
+    }
+    __syncthreads();
+    // pair p of expert e goes to slot block * (experts below e that have pairs) + (pairs of e before p);
+    // every expert holds at most `block` pairs here (a token names an expert once, tokens <= block)
+    for (int i = threadIdx.x; i < n * block; i += kRowsThreads) r_sorted[i] = n;
+    __syncthreads();
+    if (threadIdx.x < n) {
+      const int p = threadIdx.x, e = r_ids[p];
+      int rank = 0, below = 0;
+      unsigned long long seen_lo = 0, seen_hi = 0, seen_2 = 0, seen_3 = 0;  // experts < e that occur (E <= 256)
+      for (int q = 0; q < n; ++q) {
+        const int eq = r_ids[q];
+        if (eq == e && q < p) ++rank;
+        if (eq < e) {
+          unsigned long long& word = eq < 64 ? seen_lo : (eq < 128 ? seen_hi : (eq < 192 ? seen_2 : seen_3));
+          const unsigned long long bit = 1ull << (eq & 63);
+          if (!(word & bit)) { word |= bit; ++below; }
+        }
+      }
+      r_sorted[below * block + rank] = p;
+      if (rank == 0) r_expert[below] = e;
+    }
+    if (threadIdx.x == 0) {  // blocks = distinct experts
+      int blocks = 0;
+      unsigned long long s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+      for (int q = 0; q < n; ++q) {
+        const int eq = r_ids[q];
+        unsigned long long& word = eq < 64 ? s0 : (eq < 128 ? s1 : (eq < 192 ? s2 : s3));
+        const unsigned long long bit = 1ull << (eq & 63);
+        if (!(word & bit)) { word |= bit; ++blocks; }
+      }
+      r_npost = blocks * block;
+    }
+    __syncthreads();
+    npost = r_npost;
+    if (blockIdx.x == 0 && blockIdx.y == 0) {  // the arrays the down projection reads
+      for (int i = threadIdx.x; i < n; i += kRowsThreads) {
+        rt.w_out[i] = r_w[i];
+        rt.ids_out[i] = r_ids[i];
+      }
+      for (int i = threadIdx.x; i < npost; i += kRowsThreads) rt.sorted_out[i] = r_sorted[i];
+      for (int i = threadIdx.x; i < npost / block; i += kRowsThreads) rt.expert_out[i] = r_expert[i];
+      if (threadIdx.x == 0) rt.npost_out[0] = npost;
+    }
+    sorted = r_sorted;
+    expert_ids = r_expert;
+  } else {
+    npost = *a.npost;
+  }
+  if (b * block >= npost) return;
   const int kch = a.K >> 3;
   const int f0 = (blockIdx.x * (kRowsThreads / kWave) + wave) * fpw;
   const int f1 = f0 + fpw < a.N ? f0 + fpw : a.N;
-  const T* wbase = static_cast<const T*>(a.W) + static_cast<int64_t>(a.expert_ids[b]) * a.w_expert_stride;
+  const T* wbase = static_cast<const T*>(a.W) + static_cast<int64_t>(expert_ids[b]) * a.w_expert_stride;
   const int rounds = kch / (kWave * CH);
   // one load for the block's ids (block <= 64): lane l of every wavefront holds slot l's
-  const int sid_l = lane < block ? a.sorted[b * block + lane] : a.num_valid;
+  const int sid_l = lane < block ? sorted[b * block + lane] : a.num_valid;
   const unsigned long long real = __ballot(sid_l < a.num_valid);
   bool used = false;
   for (int r0 = 0; r0 < block; r0 += rows) {
@@ -135,6 +238,10 @@ inline int rows_chunks(int64_t K) {
 
 // Whether the row form takes this gate/up projection: 2-byte operands, at most kRowsMax tokens,
 // routing blocks of at most 64 slots, weight rows of whole rounds, token rows that fit the LDS.
+// Whether the same launch can also do the routing (gating + sort) of the layer.
+inline bool gateup_rows_routes(int64_t M, int E, int topk, int block) {
+  return M * topk <= kRowsPairs && E <= 256 && topk <= E && M <= block && block <= 16;
+}
 inline bool gateup_rows_fits(int64_t M, int64_t K, int block, int64_t sorted_len, int elem_bytes) {
   const int64_t rows = M < block ? M : block;
   return elem_bytes == 2 && M >= 1 && M <= kRowsMax && block <= kWave && K >= kRowsMinK && rows_chunks(K) != 0 &&
@@ -142,7 +249,7 @@ inline bool gateup_rows_fits(int64_t M, int64_t K, int block, int64_t sorted_len
 }
 
 template <typename T>
-int launch_gateup_rows(const GemmArgs& a, int block, int64_t sorted_len, hipStream_t st) {
+int launch_gateup_rows(const GemmArgs& a, int block, int64_t sorted_len, hipStream_t st, const RowsRoute& rt = RowsRoute{}) {
   const int M = a.num_valid / a.top_k;
   const int rows = M < block ? M : block;
   // blocks that hold rows: at most one per pair and per expert
@@ -153,14 +260,16 @@ int launch_gateup_rows(const GemmArgs& a, int block, int64_t sorted_len, hipStre
   const int64_t by_fill = ceil_div(static_cast<int64_t>(a.N) * active, kRowsWaves);
   int fpw = static_cast<int>(by_bytes < by_fill ? by_bytes : by_fill);
   if (fpw < 1) fpw = 1;
+  // a block holds at least one pair: no more blocks than pairs
+  const int64_t max_blocks = sorted_len / block < a.num_valid ? sorted_len / block : a.num_valid;
   const dim3 grid(static_cast<unsigned>(ceil_div(a.N, static_cast<int64_t>(kRowsThreads / kWave) * fpw)),
-                  static_cast<unsigned>(sorted_len / block));
+                  static_cast<unsigned>(max_blocks));
   const size_t lds = static_cast<size_t>(rows) * a.K * sizeof(T);
   switch (rows_chunks(a.K)) {
-    case 8: hipLaunchKernelGGL((gateup_rows_kernel<T, 8>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw); break;
-    case 7: hipLaunchKernelGGL((gateup_rows_kernel<T, 7>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw); break;
-    case 6: hipLaunchKernelGGL((gateup_rows_kernel<T, 6>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw); break;
-    case 5: hipLaunchKernelGGL((gateup_rows_kernel<T, 5>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw); break;
+    case 8: hipLaunchKernelGGL((gateup_rows_kernel<T, 8>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw, rt); break;
+    case 7: hipLaunchKernelGGL((gateup_rows_kernel<T, 7>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw, rt); break;
+    case 6: hipLaunchKernelGGL((gateup_rows_kernel<T, 6>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw, rt); break;
+    case 5: hipLaunchKernelGGL((gateup_rows_kernel<T, 5>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw, rt); break;
     default: return fail(FR_E_SHAPE, "gate/up by rows: K=%d", a.K);
   }
   return check_launch("gateup_rows_kernel");

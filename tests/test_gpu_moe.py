@@ -650,6 +650,39 @@ def test_persistent_tiles_alternating_half_empty_and_full_blocks(native, block, 
         fr.reset_tunables()
 
 
+@pytest.mark.parametrize("E,k", [(8, 2), (64, 6), (100, 3), (256, 8), (4, 4), (16, 1)])
+@pytest.mark.parametrize("ldtype", [torch.float32, torch.bfloat16])
+def test_decode_layer_routes_inside_the_gate_up_launch(native, E, k, ldtype):
+    """Up to 4 tokens with H >= 4096: fused_moe's gate/up launch gates the tokens and sorts the pairs itself.
+    Its result must equal, bit for bit, the experts-only entry point fed with the gating kernel's weights and ids
+    (the same gating core, the same routing order), and match the oracle; exact ties in the logits included."""
+    from fast_route_amd import fused_moe, fused_experts
+    from fast_route_amd.ops.stable_route import topk_softmax
+    H, Fd, dtype = 4096, 256, torch.bfloat16
+    _, _, w1, w2 = _inputs(1, H, Fd, E, 9, dtype)
+    w1d, w2d = w1.cuda(), w2.cuda()
+    for M in (1, 2, 3, 4):
+        if M * k > 32:
+            continue
+        for renorm in (True, False):
+            _say(f"routed decode E={E} k={k} {ldtype} M={M} renorm={renorm}")
+            g = torch.Generator().manual_seed(E * 100 + k * 10 + M)
+            x = torch.randn(M, H, generator=g).to(dtype)
+            logits = torch.randn(M, E, generator=g).to(ldtype)
+            if E >= 4:
+                logits[0, : min(E, 5)] = logits[0, 0]  # a run of equal logits: lower index first
+            out = fused_moe(x.cuda(), w1d, w2d, logits.cuda(), k, renorm)
+            torch.cuda.synchronize()
+            w = torch.empty((M, k), dtype=torch.float32, device="cuda")
+            ids = torch.empty((M, k), dtype=torch.int32, device="cuda")
+            topk_softmax(w, ids, None, logits.cuda(), renormalize=renorm)
+            ow, oid = oracle.gating_topk(logits, k, renorm)
+            assert torch.equal(ids.cpu(), oid)
+            same = fused_experts(x.cuda(), w1d, w2d, w, ids)
+            assert torch.equal(out, same), "routing inside the gate/up launch differs from the routing kernels"
+            _assert_close(out, oracle.fused_moe(x, w1, w2, logits, k, renorm), dtype, f"routed decode M={M}")
+
+
 def test_random_shapes_against_oracle(native):
     """Forty seeded random layer shapes (token count, widths, expert count, top-k, dtype, renormalisation)
     against the oracle: every plan boundary gets neighbours on both sides sooner or later."""
