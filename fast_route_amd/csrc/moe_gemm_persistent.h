@@ -266,19 +266,27 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   //   FR_ABL_NOLOAD  the ring is filled once and never refilled: MFMAs + fragment reads + barriers on real data
   //   FR_ABL_NOLDS   (with NOLOAD) fragments are read once and stay in registers: MFMAs + barriers
   //   FR_ABL_NOBAR   no barrier between K tiles
+  //   FR_ABL_NOMFMA  no MFMA is issued (with NOLDS: tile loads + barriers only, the kernel as a pure stream)
+  //   FR_ABL_HOTLOAD every refill fetches one of the tile's first four K tiles again (in L2, beyond the reach of
+  //                  the 32 KB L1): the loads' own cost (issue, L2 -> LDS transfer) without the misses of L2
   // They split a launch's time into its MFMA floor, the cost of the LDS fragment reads and the cost of the tile loads.
   // load q_ of an issuing wavefront (weight-tile loads first) of K tile tile_ into ring slot slot_
+#ifdef FR_ABL_HOTLOAD
+#define FR_KOFF(tile_) (((tile_) & 3) * C::BKB)
+#else
+#define FR_KOFF(tile_) ((tile_) * C::BKB)
+#endif
 #define FR_ISSUE_REAL(SET, tile_, slot_, q_)                                                                \
   {                                                                                                         \
     const int vwi_ = wave_u + ((q_) % IW) * (NW / IW);                                                      \
     if ((q_) < WI * IW) {                                                                                   \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
           wrs##SET, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vwi_) * (kWave * 16)), \
-          16, wsrc##SET[(q_) < WI * IW ? (q_) : 0], (tile_) * C::BKB, 0, 0);                                \
+          16, wsrc##SET[(q_) < WI * IW ? (q_) : 0], FR_KOFF(tile_), 0, 0);                                      \
     } else {                                                                                                \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
           xrs##SET, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WI * IW) / IW) * NW + vwi_) * (kWave * 16)), \
-          16, xsrc##SET[(q_) < WI * IW ? 0 : (q_) - WI * IW], (tile_) * C::BKB, 0, 0);                      \
+          16, xsrc##SET[(q_) < WI * IW ? 0 : (q_) - WI * IW], FR_KOFF(tile_), 0, 0);                            \
     }                                                                                                       \
   }
 #ifdef FR_ABL_NOLOAD
@@ -304,6 +312,15 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #else
 #define FR_READ_FRAGS(sl_, ks_, fb_) FR_READ_FRAGS_REAL(sl_, ks_, fb_)
 #define FR_ABL_INIT1
+#endif
+#ifdef FR_ABL_NOMFMA
+#define FR_MFMA(j_, i_, fb_) {}
+#else
+#define FR_MFMA(j_, i_, fb_)                                                                        \
+  {                                                                                                 \
+    if constexpr (C::TILE == 32) acc[j_][i_] = E::m32(wfr[fb_][j_], xf[fb_][i_], acc[j_][i_]);      \
+    else acc[j_][i_] = E::m16(wfr[fb_][j_], xf[fb_][i_], acc[j_][i_]);                              \
+  }
 #endif
 #ifdef FR_ABL_NOBAR
 #define FR_KT_BARRIER
@@ -339,8 +356,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     const int fbc = SINGLE ? 0 : (fb_);                                                       \
     _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                          \
       const int j = m / C::IT, i = m % C::IT;                                                 \
-      if constexpr (C::TILE == 32) acc[j][i] = E::m32(wfr[fbc][j], xf[fbc][i], acc[j][i]);    \
-      else acc[j][i] = E::m16(wfr[fbc][j], xf[fbc][i], acc[j][i]);                            \
+      FR_MFMA(j, i, fbc)                                                                      \
       __builtin_amdgcn_sched_barrier(0);                                                      \
       if (HAVE_NEXT) {                                                                        \
         if constexpr (SINGLE) {                                                               \
@@ -467,6 +483,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #undef FR_ISSUE_REAL
 #undef FR_READ_FRAGS_REAL
 #undef FR_ABL_INIT1
+#undef FR_KOFF
+#undef FR_MFMA
 #undef FR_KT_BARRIER
 #undef FR_MAKE_SET
 #undef FR_SLOT_ROW
