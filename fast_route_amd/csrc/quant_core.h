@@ -75,4 +75,54 @@ __device__ __forceinline__ void quant_row(const T* __restrict__ xr, int K, unsig
   }
 }
 
+// The same result from one read of the row, by a workgroup of NW wavefronts: the row's K <= 512 * NW * NC
+// elements stay in registers (NC 16-byte chunks per thread, chunk c * 64 * NW + tid: every load and every
+// 8-byte store of a wavefront is contiguous) between the reduction and the conversion; all NC loads of a
+// thread are in flight at once, and the wavefronts' maxima meet in `red` (NW floats of LDS).
+template <typename T, int NC, int NW>
+__device__ __forceinline__ void quant_row_block(const T* __restrict__ xr, int K, unsigned char* __restrict__ qr,
+                                                float* __restrict__ scale_out, int tid, float* red) {
+  typedef typename Vec8<T>::type vec8;
+  vec8 v[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int k = (c * kWave * NW + tid) * 8;
+    if (k < K) v[c] = *reinterpret_cast<const vec8*>(xr + k);
+    else v[c] = vec8{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int c = 0; c < NC; ++c)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(static_cast<float>(v[c][i])));
+  amax = wave_max(amax);
+  if (tid % kWave == 0) red[tid / kWave] = amax;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < NW; ++w) amax = fmaxf(amax, red[w]);
+  const float s = amax > 0.f ? amax / 448.f : 1.f;
+  if (tid == 0) *scale_out = s;
+  const bool fast = amax >= 0x1p-40f && amax <= 0x1p40f;  // see quant_row
+  const float y = 1.f / s;
+  auto quot = [&](float x) {
+    if (fast) {
+      const float q0 = x * y;
+      const float r = __builtin_fmaf(-s, q0, x);
+      return __builtin_fmaf(r, y, q0);
+    }
+    return x / s;
+  };
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int k = (c * kWave * NW + tid) * 8;
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = fminf(fmaxf(quot(static_cast<float>(v[c][i])), -448.f), 448.f);
+    uint2 o;
+    o.x = pack4(f[0], f[1], f[2], f[3]);
+    o.y = pack4(f[4], f[5], f[6], f[7]);
+    if (k < K) *reinterpret_cast<uint2*>(qr + k) = o;
+  }
+}
+
 }  // namespace fr
