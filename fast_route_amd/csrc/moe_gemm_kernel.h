@@ -168,7 +168,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_rsrc(const T* p) {
 }
 #endif
 
-template <typename T, typename C, int EPI, typename AccT>
+template <typename T, typename C, int EPI, bool HOIST = true, typename AccT>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::JF][C::IT], int pid_t, int pid_f,
                                               int expert, int split, int wt, int wf, int frow, int kgrp) {
   typedef Elem<T> E;
@@ -181,18 +181,69 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
   // group g (TILE==32: 4 groups of 4 regs; TILE==16: one), 4 consecutive features
   // starting at g*8 + kgrp*4 (TILE==32) or kgrp*4 (TILE==16) inside the MFMA tile.
   constexpr int GROUPS = ACC_N / 4;
+  // fp8: with HOIST the scales of the lane's weight rows (the same for every token tile) and of its token rows
+  // are fetched up front, all loads in flight together, instead of one by one between the stores (which the
+  // compiler may not move them across).  That takes JF * ACC_N registers: the persistent kernel, which keeps
+  // two address sets alive across its epilogue, does without.
+  constexpr int NWS = (E::SCALED && HOIST) ? C::JF * GROUPS * 4 : 1;
+  float wscale[NWS];
+  float xscale[C::IT];
+  int sids[C::IT];
+#pragma unroll
+  for (int i = 0; i < C::IT; ++i) {
+    sids[i] = 0;
+    xscale[i] = 1.f;
+  }
+  if constexpr (EPI != EPI_SILU || E::SCALED) {
+#pragma unroll
+    for (int i = 0; i < C::IT; ++i) sids[i] = a.sorted[pid_t * BT + wt * C::TT + i * C::TILE + frow];
+  }
+  float routed[C::IT];  // routed weight of the lane's pair in each token tile (all fetched before the first store)
+#pragma unroll
+  for (int i = 0; i < C::IT; ++i) {
+    routed[i] = 1.f;
+    if constexpr (EPI != EPI_SILU)
+      if (a.mul_weight && sids[i] < a.num_valid) routed[i] = a.topk_w[sids[i]];
+  }
   const float* wsc = nullptr;
   if constexpr (E::SCALED) wsc = a.w_scale + static_cast<int64_t>(expert) * a.w_rows;
+  // scale of the weight row behind accumulator register (j, g, r)
+  auto w_scale_at = [&](int j, int g, int r) -> float {
+    int f;
+    if constexpr (EPI == EPI_SILU) {
+      constexpr int HJ = C::JF / 2;
+      const int fl = pid_f * (BF / 2) + wf * (C::TF / 2) + (j % HJ) * C::TILE + g * 8 + kgrp * 4 + r;
+      f = (j / HJ) * a.N + (fl < a.N ? fl : a.N - 1);
+    } else {
+      const int fl = pid_f * BF + wf * C::TF + j * C::TILE + g * 8 + kgrp * 4 + r;
+      f = fl < a.N ? fl : a.N - 1;
+    }
+    return wsc[f];
+  };
+  auto w_scale = [&](int j, int g, int r) -> float {
+    if constexpr (HOIST) return wscale[(j * GROUPS + g) * 4 + r];
+    else return w_scale_at(j, g, r);
+  };
+  if constexpr (E::SCALED) {
+    if constexpr (HOIST) {
+#pragma unroll
+      for (int j = 0; j < C::JF; ++j)
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) wscale[(j * GROUPS + g) * 4 + r] = w_scale_at(j, g, r);
+    }
+#pragma unroll
+    for (int i = 0; i < C::IT; ++i) {
+      if (a.top_k > 0) xscale[i] = sids[i] < a.num_valid ? a.x_scale[sids[i] / a.top_k] : 1.f;
+      else xscale[i] = a.x_scale[pid_t * BT + wt * C::TT + i * C::TILE + frow];
+    }
+  }
 #pragma unroll
   for (int i = 0; i < C::IT; ++i) {
     const int slot = pid_t * BT + wt * C::TT + i * C::TILE + frow;
-    int sid = 0;
-    if constexpr (EPI != EPI_SILU || E::SCALED) sid = a.sorted[slot];
-    float xs = 1.f;
-    if constexpr (E::SCALED) {
-      if (a.top_k > 0) xs = sid < a.num_valid ? a.x_scale[sid / a.top_k] : 1.f;
-      else xs = a.x_scale[slot];
-    }
+    const int sid = sids[i];
+    const float xs = xscale[i];
     if constexpr (EPI == EPI_SILU) {
       constexpr int HJ = C::JF / 2;
       out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(slot) * a.ldo;
@@ -206,9 +257,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
           for (int r = 0; r < 4; ++r) {
             float gv = acc[j][i][g * 4 + r], uv = acc[j + HJ][i][g * 4 + r];
             if constexpr (E::SCALED) {
-              const int fc = f + r < a.N ? f + r : a.N - 1;
-              gv *= xs * wsc[fc];
-              uv *= xs * wsc[a.N + fc];
+              gv *= xs * w_scale(j, g, r);
+              uv *= xs * w_scale(j + HJ, g, r);
             }
             o[r] = static_cast<out_t>(silu(gv) * uv);
           }
@@ -219,7 +269,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
         }
     } else {
       if (sid < a.num_valid) {
-        const float rw = (a.mul_weight ? a.topk_w[sid] : 1.f) * xs;
+        const float rw = routed[i] * xs;
 #pragma unroll
         for (int j = 0; j < C::JF; ++j)
 #pragma unroll
@@ -229,7 +279,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               v[r] = acc[j][i][g * 4 + r] * rw;
-              if constexpr (E::SCALED) v[r] *= wsc[f + r < a.N ? f + r : a.N - 1];
+              if constexpr (E::SCALED) v[r] *= w_scale(j, g, r);
             }
             if constexpr (EPI == EPI_DOWN) {
               float* orow = static_cast<float*>(a.out) + static_cast<int64_t>(split) * a.split_stride +

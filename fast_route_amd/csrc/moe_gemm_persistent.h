@@ -151,6 +151,10 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, IW = C::IW, NLI = (XI + WI) * IW;
   constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
   constexpr bool SINGLE = E::SCALED;   // one fragment buffer for fp8 (8-register fragments), two otherwise
+  // fp8 epilogue: scales fetched up front where the registers allow it (the 256-row tile keeps 128 accumulators
+  // and two address sets alive: measured 603 us with, 589 us without for the down projection at M = 4096; the
+  // 128-row tile gains 2-5 %)
+  constexpr bool HOIST = BT < 256;
   static_assert(S >= 2 && C::SPREAD <= 1, "persistent form: ring of at least two slots, refill in one group");
   static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
   static_assert((S - 1) * NLI <= 63, "vmcnt budget");
@@ -440,7 +444,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
       for (int kt = 0; kt < S - 1; ++kt) FR_KTILE(ISS_, false, A, 0, false, 0)                             \
       FR_KTILE(ISS_, false, A, 0, true, 0)                                                                 \
     }                                                                                                      \
-    if (tu < 0) gemm_epilogue<T, C, EPI>(a, acc, pid_t, pid_f, expert, split, wt, wf, frow, kgrp);         \
+    if (tu < 0) gemm_epilogue<T, C, EPI, HOIST>(a, acc, pid_t, pid_f, expert, split, wt, wf, frow, kgrp);         \
     else tail_store<C, EPI>(a.tail_ws + static_cast<int64_t>(xcd * nper + tu) * (BT * BF), acc, wt, wf, frow, kgrp); \
   }
   // Fill of the ring with the first S K tiles of set A and the first fragments.

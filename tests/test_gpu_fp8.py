@@ -19,7 +19,10 @@ def _say(msg):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_row_quantisation_bit_exact(native, dtype):
     from fast_route_amd import quantize_rows_e4m3
-    for rows, K, std in ((1, 16, 1.0), (37, 1024, 1.0), (130, 4096, 0.02), (16, 14336, 3.0)):
+    # rows of up to 16384 elements are held in registers by a workgroup (2, 4 or 8 chunks per thread, the last
+    # one partly filled); longer rows take the two-pass kernel
+    for rows, K, std in ((1, 16, 1.0), (37, 1024, 1.0), (130, 4096, 0.02), (16, 14336, 3.0), (9, 5008, 1.0),
+                         (3, 9008, 0.5), (4, 16384, 1.0), (5, 16400, 1.0)):
         _say(f"quant rows={rows} K={K} std={std} {dtype}")
         g = torch.Generator().manual_seed(rows * 7 + K)
         x = (torch.randn(rows, K, generator=g) * std).to(dtype)
