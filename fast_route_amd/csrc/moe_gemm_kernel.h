@@ -110,7 +110,9 @@ template <> struct Elem<fp8_t> {
   }
 };
 
-__device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); }
+// g * sigmoid(g).  The quotient is a multiplication by v_rcp_f32 (1 ulp) instead of the IEEE division's ten
+// instructions: the result is rounded to 8 or 11 bits right after, and the epilogue's VALU time is MFMA idle time.
+__device__ __forceinline__ float silu(float g) { return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)); }
 
 // Tile configuration.  BKB = bytes of K per row per tile (64 bf16 or 128 fp8 = 128 B,
 // the L2 line: shorter row segments halve the L2->LDS rate).  TILE = 32 uses the
