@@ -123,7 +123,10 @@ int gateup_impl(const void* x, const float* x_scale, const void* w1, const float
   a.num_valid = (int)n; a.top_k = topk; a.N = (int)F; a.K = (int)H;
   a.num_experts = E;
   a.tail_ws = tail_ws;
-  if (gateup_rows_fits(M, H, block, sorted_len, elem_bytes(dtype))) {
+  // batches the routed form of the row kernel takes run the row kernel here too (same kernel, same sums, whoever
+  // did the routing)
+  const int64_t min_k = gateup_rows_routes(M, E, topk, block) ? kRowsMinKRouted : kRowsMinK;
+  if (gateup_rows_fits(M, H, block, sorted_len, elem_bytes(dtype), min_k)) {
     // a handful of tokens: stream the weight rows past the token rows without tiles
     if (dtype == FR_BF16) return launch_gateup_rows<bf16_t>(a, block, sorted_len / block * block, st);
     return launch_gateup_rows<f16_t>(a, block, sorted_len / block * block, st);
@@ -135,7 +138,7 @@ int gateup_rows_routed(const void* x, const void* w1, const void* logits, int lo
                        int64_t F, int E, int topk, int renorm, int block, int dtype, void* act, float* topk_w,
                        int32_t* topk_ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, hipStream_t st) {
   const int64_t n = M * topk, sorted_len = n + int64_t(E) * (block - 1);
-  if ((dtype != FR_BF16 && dtype != FR_F16) || !gateup_rows_fits(M, H, block, sorted_len, 2) ||
+  if ((dtype != FR_BF16 && dtype != FR_F16) || !gateup_rows_fits(M, H, block, sorted_len, 2, kRowsMinKRouted) ||
       !gateup_rows_routes(M, E, topk, block) || F % 8 != 0 ||
       (logits_dtype != FR_F32 && logits_dtype != FR_F16 && logits_dtype != FR_BF16))
     return 1;

@@ -22,6 +22,7 @@ namespace fr {
 constexpr int kRowsMax = 4;        // tokens in the batch (hence token rows per pass over a routing block) the row form takes
 constexpr int kRowsThreads = 256;  // 4 wavefronts
 constexpr int kRowsMinK = 4096;    // shorter rows: the tile kernel is as fast (measured at 1024 and 2048)
+constexpr int kRowsMinKRouted = 2048;  // ... unless this launch also does the routing: one launch less ahead of it
 constexpr int kRowsWaves = 4096;   // wavefronts the feature runs are cut for: 16 on each of 256 CUs
 constexpr int kRowsWaveBytes = 7 * 16384;  // weight bytes a wavefront streams
 constexpr int kRowsLds = 62464;    // token rows in LDS: the default limit of 64 KB less the kernel's static arrays
@@ -92,7 +93,7 @@ __device__ __forceinline__ void rows_gate(const LT* logits, int M, int E, int to
 }
 
 // CH = 16-byte chunks per lane, row and round: a weight row is `rounds` x CH x 512 elements (CH = 8 for K = 4096
-// and 8192, 5 for 5120, 6 for 6144, 7 for 7168); a lane has 2 * CH loads in flight.
+// and 8192, 5 for 5120, 6 for 6144, 7 for 7168, 4 for 2048); a lane has 2 * CH loads in flight.
 // grid.x * 4 wavefronts cover the F features in runs of `fpw`; grid.y = routing blocks (upper bound).
 // A block's slots are taken `rows` at a time (rows = tokens in the batch <= kRowsMax): a token
 // selects an expert once, so all rows of a block are in its first pass and the later passes find
@@ -227,11 +228,11 @@ __global__ void __launch_bounds__(kRowsThreads) gateup_rows_kernel(GemmArgs a, i
   }
 }
 
-// Chunks per round for rows of K elements: the largest of 8..5 that divides K / 512, or 0.
+// Chunks per round for rows of K elements: the largest of 8..4 that divides K / 512, or 0.
 inline int rows_chunks(int64_t K) {
   if (K % 512 != 0) return 0;
   const int64_t nc = K / 512;
-  for (int ch = 8; ch >= 5; --ch)
+  for (int ch = 8; ch >= 4; --ch)
     if (nc % ch == 0) return ch;
   return 0;
 }
@@ -242,9 +243,9 @@ inline int rows_chunks(int64_t K) {
 inline bool gateup_rows_routes(int64_t M, int E, int topk, int block) {
   return M * topk <= kRowsPairs && E <= 256 && topk <= E && M <= block && block <= 16;
 }
-inline bool gateup_rows_fits(int64_t M, int64_t K, int block, int64_t sorted_len, int elem_bytes) {
+inline bool gateup_rows_fits(int64_t M, int64_t K, int block, int64_t sorted_len, int elem_bytes, int64_t min_k = kRowsMinK) {
   const int64_t rows = M < block ? M : block;
-  return elem_bytes == 2 && M >= 1 && M <= kRowsMax && block <= kWave && K >= kRowsMinK && rows_chunks(K) != 0 &&
+  return elem_bytes == 2 && M >= 1 && M <= kRowsMax && block <= kWave && K >= min_k && rows_chunks(K) != 0 &&
          rows * K * 2 <= kRowsLds && sorted_len / block <= 65535;  // routing blocks are the grid's y dimension
 }
 
@@ -270,6 +271,7 @@ int launch_gateup_rows(const GemmArgs& a, int block, int64_t sorted_len, hipStre
     case 7: hipLaunchKernelGGL((gateup_rows_kernel<T, 7>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw, rt); break;
     case 6: hipLaunchKernelGGL((gateup_rows_kernel<T, 6>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw, rt); break;
     case 5: hipLaunchKernelGGL((gateup_rows_kernel<T, 5>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw, rt); break;
+    case 4: hipLaunchKernelGGL((gateup_rows_kernel<T, 4>), grid, dim3(kRowsThreads), lds, st, a, block, rows, fpw, rt); break;
     default: return fail(FR_E_SHAPE, "gate/up by rows: K=%d", a.K);
   }
   return check_launch("gateup_rows_kernel");
