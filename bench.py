@@ -309,15 +309,19 @@ def cpu_baseline(torch, shape, layer, sample_tokens):
     m = min(sample_tokens, layer.M)
     x, logits = layer.x[:m].cpu(), layer.logits[:m].cpu()
     w1, w2 = layer.w1.cpu(), layer.w2.cpu()
-    t0 = time.perf_counter()
-    ref = oracle.fused_moe(x, w1, w2, logits, shape["topk"], True)
-    dt = time.perf_counter() - t0
+    times, spent = [], 0.0
+    while len(times) < 3 and spent < 12.0:  # a bounded sample: up to three passes, about 10 s of CPU work
+        t0 = time.perf_counter()
+        ref = oracle.fused_moe(x, w1, w2, logits, shape["topk"], True)
+        times.append(time.perf_counter() - t0)
+        spent += times[-1]
+    dt = sorted(times)[len(times) // 2]
     got = layer.out[:m].float().cpu()
     err = (got - ref).abs().max().item()
     return {"value": round(layer_flops(m, shape["H"], shape["F"], shape["topk"]) / dt / 1e12, 4), "unit": "TFLOP/s",
             "cores": threads, "kind": "port", "cpu_model": model, "host_cpus": os.cpu_count(),
-            "sample": "fp32 PyTorch oracle, first %d tokens of the M=%d batch, weights upcast per expert, 1 rep, %.1f s"
-                      % (m, layer.M, dt),
+            "sample": "fp32 PyTorch oracle, first %d tokens of the M=%d batch, weights upcast per expert, median of %d passes, %.1f s each"
+                      % (m, layer.M, len(times), dt),
             "us_per_layer_sample": round(dt * 1e6, 0), "max_abs_err_vs_gpu": err,
             "ref_max_abs": ref.abs().max().item()}
 
@@ -478,7 +482,7 @@ def main():
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="skip the small / routing / fine-grained / fp8 records")
-    ap.add_argument("--cpu-tokens", type=int, default=1024)
+    ap.add_argument("--cpu-tokens", type=int, default=4096)
     ap.add_argument("--routing", action="store_true", help="also time the routing-only stress workload")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB device copy: the kernel of known size that calibrates "
