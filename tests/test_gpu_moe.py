@@ -692,7 +692,7 @@ def test_random_shapes_against_oracle(native):
     for case in range(40):
         E = int(rng.choice([1, 2, 3, 4, 8, 16, 60, 64]))
         k = int(rng.integers(1, min(E, 8) + 1))
-        H = int(rng.choice([128, 256, 384, 512, 1024, 4096]))
+        H = int(rng.choice([128, 256, 384, 512, 1024, 2048, 3072, 4096]))
         Fd = int(rng.choice([128, 256, 384, 640]))
         M = int(rng.choice([1, 2, 3, 4, 5, 7, 17, 33, 100, 257, 600]) if rng.random() < 0.7 else rng.integers(1, 700))
         dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
