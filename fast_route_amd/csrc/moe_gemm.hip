@@ -8,26 +8,29 @@ namespace fr {
 // P = float (one fp32 slice per K split) or the operand type (single slice: each pair's row
 // rounded once before the sum over its token's slots, as the reference's second GEMM writes it,
 // fast_route/fast_route/ops/fused_moe.py:117-123, before torch.sum).
-template <typename T, typename P>
+template <typename T, typename P, int V>
 __global__ __launch_bounds__(256) void combine_kernel(const P* __restrict__ partial,
                                                       int64_t split_stride, int splits, int topk,
                                                       int64_t M, int H, T* __restrict__ out) {
-  typedef P p4 __attribute__((ext_vector_type(4)));
-  const int64_t idx = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  typedef P pv __attribute__((ext_vector_type(V)));
+  typedef T tv __attribute__((ext_vector_type(V)));
+  const int64_t idx = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * V;
   if (idx >= M * H) return;
   const int64_t m = idx / H;
   const int h = static_cast<int>(idx % H);
-  f32x4 s = {0.f, 0.f, 0.f, 0.f};
+  float s[V];
+#pragma unroll
+  for (int r = 0; r < V; ++r) s[r] = 0.f;
   for (int j = 0; j < topk; ++j)
     for (int sp = 0; sp < splits; ++sp) {
-      const p4 v = *reinterpret_cast<const p4*>(partial + sp * split_stride + (m * topk + j) * H + h);
+      const pv v = *reinterpret_cast<const pv*>(partial + sp * split_stride + (m * topk + j) * H + h);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) s[r] += static_cast<float>(v[r]);
+      for (int r = 0; r < V; ++r) s[r] += static_cast<float>(v[r]);
     }
-  typename Elem<T>::out4 o;
+  tv o;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) o[r] = static_cast<T>(s[r]);
-  *reinterpret_cast<typename Elem<T>::out4*>(out + idx) = o;
+  for (int r = 0; r < V; ++r) o[r] = static_cast<T>(s[r]);
+  *reinterpret_cast<tv*>(out + idx) = o;
 }
 
 // ---- tile launches: instantiated per (element type, epilogue) in moe_gemm_inst_*.hip ---------
@@ -57,8 +60,15 @@ int dispatch_dtype(const GemmArgs& a, int dtype, int block, int splits, int64_t 
 template <typename T, typename P>
 void launch_combine_as(const void* partial, int64_t split_stride, int splits, int topk, int64_t M, int H, void* out,
                        hipStream_t st) {
+  // 16-byte loads of the 2-byte rows of a single slice when the row length allows, else 4 elements per thread
+  if (sizeof(P) == 2 && H % 8 == 0) {
+    const unsigned grid = static_cast<unsigned>(ceil_div(M * H / 8, 256));
+    hipLaunchKernelGGL((combine_kernel<T, P, 8>), dim3(grid), dim3(256), 0, st, static_cast<const P*>(partial), split_stride,
+                       splits, topk, M, H, static_cast<T*>(out));
+    return;
+  }
   const unsigned grid = static_cast<unsigned>(ceil_div(M * H / 4, 256));
-  hipLaunchKernelGGL((combine_kernel<T, P>), dim3(grid), dim3(256), 0, st, static_cast<const P*>(partial), split_stride,
+  hipLaunchKernelGGL((combine_kernel<T, P, 4>), dim3(grid), dim3(256), 0, st, static_cast<const P*>(partial), split_stride,
                      splits, topk, M, H, static_cast<T*>(out));
 }
 
