@@ -3,7 +3,7 @@
 // (moe_gemm_inst_*.hip) so that the library builds in parallel; moe_gemm.hip sees only
 // the declaration of dispatch_block.
 #pragma once
-#include "moe_gemm_persistent.h"
+#include "moe_gemm_quad.h"
 
 namespace fr {
 
@@ -69,7 +69,15 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       // epilogue: the hand-off K tiles spill; without the hand-off it is within 1 % of the plain kernel),
       // which keeps the plain kernel.
       if constexpr (sizeof(T) == 1 && EPI == EPI_SILU) return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
-      else return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
+      else {
+#ifdef FR_QUAD
+        if constexpr (sizeof(T) == 2) {
+          const int rc = launch_gemm_quad<T, EPI>(a, splits, st);
+          if (rc != 1) return rc;
+        }
+#endif
+        return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
+      }
     case 128:
       fill(128, TL::T128::BF, TL::T128::BKB);
       // The gate/up GEMM always takes the persistent form (its walk by expert fetches each expert's

@@ -121,12 +121,15 @@ __global__ void __launch_bounds__(kRowsThreads) gateup_rows_kernel(GemmArgs a, i
     // every expert holds at most `block` pairs here (a token names an expert once, tokens <= block)
     for (int i = threadIdx.x; i < n * block; i += kRowsThreads) r_sorted[i] = n;
     __syncthreads();
+    // An id outside [0, E) (a token row of NaN logits can leave one behind) is a dropped pair, as in the
+    // routing kernels: no slot, no block, never an index into the weights.
     if (threadIdx.x < n) {
       const int p = threadIdx.x, e = r_ids[p];
       int rank = 0, below = 0;
       unsigned long long seen_lo = 0, seen_hi = 0, seen_2 = 0, seen_3 = 0;  // experts < e that occur (E <= 256)
       for (int q = 0; q < n; ++q) {
         const int eq = r_ids[q];
+        if (eq < 0 || eq >= rt.E) continue;
         if (eq == e && q < p) ++rank;
         if (eq < e) {
           unsigned long long& word = eq < 64 ? seen_lo : (eq < 128 ? seen_hi : (eq < 192 ? seen_2 : seen_3));
@@ -134,14 +137,17 @@ __global__ void __launch_bounds__(kRowsThreads) gateup_rows_kernel(GemmArgs a, i
           if (!(word & bit)) { word |= bit; ++below; }
         }
       }
-      r_sorted[below * block + rank] = p;
-      if (rank == 0) r_expert[below] = e;
+      if (e >= 0 && e < rt.E) {
+        r_sorted[below * block + rank] = p;
+        if (rank == 0) r_expert[below] = e;
+      }
     }
     if (threadIdx.x == 0) {  // blocks = distinct experts
       int blocks = 0;
       unsigned long long s0 = 0, s1 = 0, s2 = 0, s3 = 0;
       for (int q = 0; q < n; ++q) {
         const int eq = r_ids[q];
+        if (eq < 0 || eq >= rt.E) continue;
         unsigned long long& word = eq < 64 ? s0 : (eq < 128 ? s1 : (eq < 192 ? s2 : s3));
         const unsigned long long bit = 1ull << (eq & 63);
         if (!(word & bit)) { word |= bit; ++blocks; }
@@ -168,7 +174,9 @@ __global__ void __launch_bounds__(kRowsThreads) gateup_rows_kernel(GemmArgs a, i
   const int kch = a.K >> 3;
   const int f0 = (blockIdx.x * (kRowsThreads / kWave) + wave) * fpw;
   const int f1 = f0 + fpw < a.N ? f0 + fpw : a.N;
-  const T* wbase = static_cast<const T*>(a.W) + static_cast<int64_t>(expert_ids[b]) * a.w_expert_stride;
+  const int expert = expert_ids[b];
+  if (expert < 0 || expert >= a.num_experts) return;  // never form a weight address from an id the routing did not vouch for
+  const T* wbase = static_cast<const T*>(a.W) + static_cast<int64_t>(expert) * a.w_expert_stride;
   const int rounds = kch / (kWave * CH);
   // one load for the block's ids (block <= 64): lane l of every wavefront holds slot l's
   const int sid_l = lane < block ? sorted[b * block + lane] : a.num_valid;
