@@ -104,7 +104,7 @@ int64_t tail_scratch_bytes(int block, int dtype, int64_t K, int64_t N, bool gate
   // The tiles that run persistently: T256 (both GEMMs for 2-byte operands, the down projection for fp8)
   // and T128P (both GEMMs).  Same K bytes per tile and same feature tile in all of them.
   typedef Tiles<bf16_t>::T256 C;
-  static_assert(Tiles<bf16_t>::T128P::BF == C::BF && Tiles<bf16_t>::T128P::BKB == C::BKB, "same K tile and feature tile");
+  static_assert(Tiles<bf16_t>::T256S::BF == C::BF && Tiles<bf16_t>::T256S::BT == C::BT && Tiles<bf16_t>::T128P::BF == C::BF && Tiles<bf16_t>::T128P::BKB == C::BKB, "same K tile and feature tile");
   static_assert(Tiles<fp8_t>::T256::BF == C::BF && Tiles<fp8_t>::T256::BKB == C::BKB, "same K tile and feature tile");
   const bool two_byte = dtype == FR_BF16 || dtype == FR_F16;
   if (!two_byte && dtype != FR_FP8_E4M3) return 0;
@@ -295,3 +295,8 @@ extern "C" int fr_moe_prepare(int dtype) {
   }
   return rc;
 }
+
+#ifdef FR_PROF
+// measurement builds only: device buffer of 4 x int64 per workgroup the persistent kernels leave their cycle counts in
+extern "C" void fr_debug_set_prof(long long* p) { fr::fr_prof_host() = p; }
+#endif

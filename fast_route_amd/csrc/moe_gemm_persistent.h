@@ -137,8 +137,16 @@ __device__ __forceinline__ void tail_store(float* tile, AccT (&acc)[C::JF][C::IT
   }
 }
 
+#ifdef FR_PROF  // measurement builds: cycle counts of wavefront 0 of every workgroup (K loops / epilogues / total / K tiles)
+#define FR_PROF_PARAM , long long* fr_prof_buf
+#define FR_PROF_ARG , fr_prof_host()
+inline long long*& fr_prof_host() { static long long* p = nullptr; return p; }
+#else
+#define FR_PROF_PARAM
+#define FR_PROF_ARG
+#endif
 template <typename T, typename C, int EPI>
-__global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(const GemmArgs a) {
+__global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(const GemmArgs a FR_PROF_PARAM) {
 #if defined(__HIP_DEVICE_COMPILE__)  // buffer resources and LDS-DMA builtins exist in the device pass only
   typedef Elem<T> E;
   typedef typename std::conditional<C::TILE == 32, f32x16, f32x4>::type acc_t;
@@ -150,13 +158,15 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
   constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, IW = C::IW, NLI = (XI + WI) * IW;
   constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
-  constexpr bool SINGLE = E::SCALED;   // one fragment buffer for fp8 (8-register fragments), two otherwise
+  // one fragment buffer for fp8 (8-register fragments) and for the 256-row tile on 16x16 MFMAs (twelve fragments
+  // per K-step next to 128 accumulators), two otherwise
+  constexpr bool SINGLE = E::SCALED || (C::TILE == 16 && BT == 256);
   // fp8 epilogue: scales fetched up front where the registers allow it (the 256-row tile keeps 128 accumulators
   // and two address sets alive: measured 603 us with, 589 us without for the down projection at M = 4096; the
   // 128-row tile gains 2-5 %)
   constexpr bool HOIST = BT < 256;
   static_assert(S >= 2 && C::SPREAD <= 1, "persistent form: ring of at least two slots, refill in one group");
-  static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
+  static_assert(SINGLE || KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
   static_assert((S - 1) * NLI <= 63, "vmcnt budget");
   static_assert(EPI != EPI_SILU || C::JF % 2 == 0, "gate and up tiles must pair up inside a wave");
   static_assert(IW >= 1 && NW % IW == 0, "issue width");
@@ -318,12 +328,12 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #define FR_ABL_INIT1
 #endif
 #ifdef FR_ABL_NOMFMA
-#define FR_MFMA(j_, i_, fb_) {}
+#define FR_MFMA(j_, i_, fbw_, fbx_) {}
 #else
-#define FR_MFMA(j_, i_, fb_)                                                                        \
+#define FR_MFMA(j_, i_, fbw_, fbx_)                                                                 \
   {                                                                                                 \
-    if constexpr (C::TILE == 32) acc[j_][i_] = E::m32(wfr[fb_][j_], xf[fb_][i_], acc[j_][i_]);      \
-    else acc[j_][i_] = E::m16(wfr[fb_][j_], xf[fb_][i_], acc[j_][i_]);                              \
+    if constexpr (C::TILE == 32) acc[j_][i_] = E::m32(wfr[fbw_][j_], xf[fbx_][i_], acc[j_][i_]);    \
+    else acc[j_][i_] = E::m16(wfr[fbw_][j_], xf[fbx_][i_], acc[j_][i_]);                            \
   }
 #endif
 #ifdef FR_ABL_NOBAR
@@ -360,7 +370,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     const int fbc = SINGLE ? 0 : (fb_);                                                       \
     _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                          \
       const int j = m / C::IT, i = m % C::IT;                                                 \
-      FR_MFMA(j, i, fbc)                                                                      \
+      FR_MFMA(j, i, fbc, fbc)                                                                 \
       __builtin_amdgcn_sched_barrier(0);                                                      \
       if (HAVE_NEXT) {                                                                        \
         if constexpr (SINGLE) {                                                               \
@@ -407,6 +417,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   // refill the ring during the last S K tiles of this one.
 #define FR_TILE(ISS_, NEXT)                                                                                \
   {                                                                                                        \
+    FR_STAMP(0)                                                                                            \
     /* A wavefront that issues no loads and whose token rows of this block are all padding (the upper */   \
     /* half of a block that holds at most half a block of pairs) has nothing to multiply: it keeps the */  \
     /* barriers and leaves the MFMA pipe and the LDS to the wavefront it shares the SIMD with.  When */     \
@@ -444,6 +455,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
       for (int kt = 0; kt < S - 1; ++kt) FR_KTILE(ISS_, false, A, 0, false, 0)                             \
       FR_KTILE(ISS_, false, A, 0, true, 0)                                                                 \
     }                                                                                                      \
+    FR_STAMP(1)                                                                                            \
     if (tu < 0) gemm_epilogue<T, C, EPI, HOIST>(a, acc, pid_t, pid_f, expert, split, wt, wf, frow, kgrp);         \
     else tail_store<C, EPI>(a.tail_ws + static_cast<int64_t>(xcd * nper + tu) * (BT * BF), acc, wt, wf, frow, kgrp); \
   }
@@ -471,8 +483,27 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
       _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) wsrcA[ih] = wsrcB[ih];                        \
     }                                                                                                      \
     FR_TILE(ISS_, false)                                                                                   \
+    FR_STAMP(2)                                                                                            \
   }
+#ifdef FR_PROF
+  long long pf_t[2] = {0, 0}, pf_last = __builtin_readcyclecounter(), pf_periods = 0;
+  const long long pf_begin = pf_last;
+#define FR_STAMP(k_)                                                                   \
+  {                                                                                    \
+    const long long n_ = __builtin_readcyclecounter();                                 \
+    pf_t[(k_) == 1 ? 0 : 1] += n_ - pf_last;                                           \
+    pf_last = n_;                                                                      \
+    if ((k_) == 1) pf_periods += kn;                                                   \
+    if ((k_) == 2 && threadIdx.x == 0 && fr_prof_buf) {                                \
+      long long* o_ = fr_prof_buf + blockIdx.x * 4;                                    \
+      o_[0] = pf_t[0]; o_[1] = pf_t[1]; o_[2] = n_ - pf_begin; o_[3] = pf_periods;     \
+    }                                                                                  \
+  }
+#else
+#define FR_STAMP(k_)
+#endif
   if (IW == 1 || issuer) FR_PERSIST(true) else FR_PERSIST(false)
+#undef FR_STAMP
 #undef FR_PERSIST
 #undef FR_FILL
 #undef FR_TILE
@@ -644,7 +675,7 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
     grid = (worst + 7) / 8 * 8;
   }
   hipLaunchKernelGGL((moe_gemm_persistent_kernel<T, C, EPI>), dim3(static_cast<unsigned>(grid), splits), dim3(C::NT),
-                     C::LDS_BYTES, st, a);
+                     C::LDS_BYTES, st, a FR_PROF_ARG);
   int lrc = check_launch("moe_gemm_persistent_kernel");
   if (lrc != FR_OK || !tail) return lrc;
   if constexpr (kFixable) {

@@ -3,7 +3,7 @@
 // (moe_gemm_inst_*.hip) so that the library builds in parallel; moe_gemm.hip sees only
 // the declaration of dispatch_block.
 #pragma once
-#include "moe_gemm_quad.h"
+#include "moe_gemm_persistent.h"
 
 namespace fr {
 
@@ -20,8 +20,15 @@ namespace fr {
 //                   segments: T32L / T16L, used when H allows.
 template <typename T> struct Tiles {  // bf16 / fp16
   typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 2> T256;
+  // The same tile on v_mfma_f32_16x16x32: half the accumulator-register traffic per flop of the 32x32x16 shape.
+  // The part's clock under MFMA load follows the power drawn: a pure stream of 16x16x32 MFMAs holds 2.0 GHz where
+  // 32x32x16 holds 1.4-1.8 GHz.  One fragment buffer (the second would not fit next to 128 accumulators and two
+  // address sets).  Gate/up at 4096 / 16384 tokens: -2.5 % / -5 %, down projection -3 % / -4 %; with a short K loop
+  // (2048: half as many K tiles to spread a tile's hand-over on) it loses 4 %, hence kSmallMfmaMinK.
+  typedef Cfg<256, 256, 128, 2, 4, 16, 1, 2, 0, 2> T256S;
+  typedef T256 T256G;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
-  typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;  // persistent form; one wavefront per SIMD issues the loads (2-4 % over each its own)
+  typedef Cfg<128, 256, 128, 2, 4, 16, 1, 3, 0, 2> T128P;  // persistent form; one wavefront per SIMD issues the loads (2-4 % over each its own); 16x16x32 MFMAs: 2-3 % over 32x32x16
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 3, 3> T64;    // 3-slot ring like the 128-row tile (5 % over the register-staged form)
   typedef Cfg<64, 128, 256, 2, 2, 32, 1, 3> T64U;      // gate/up: 256-byte row segments, 4 wavefronts (another 5 %)
   typedef Cfg<32, 128, 128, 1, 4, 16, 2, 3> T32;
@@ -33,7 +40,9 @@ template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per
   // every wavefront issues its own tile loads: half the address registers per wavefront (the persistent down
   // projection spills 16 instead of 57 registers: 586 vs 595 us at M=4096 although no wavefront can then skip an
   // all-padding half tile; the plain gate/up kernel is unchanged)
+  typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 1> T256G;  // gate/up GEMM (plain kernel, two fragment buffers)
   typedef Cfg<256, 256, 128, 2, 4, 32, 1, 2, 0, 1> T256;
+  typedef T256 T256S;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 3, 3> T64;
@@ -43,6 +52,8 @@ template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per
   typedef Cfg<32, 128, 512, 1, 4, 16, 1, 2> T32L;
   typedef Cfg<16, 64, 512, 1, 2, 16, 2, 2> T16L;
 };
+
+constexpr int kSmallMfmaMinK = 4096;  // K from which the 256-row tile of 2-byte operands takes the 16x16x32 MFMA form
 
 inline bool valid_block(int block) { return block == 16 || block == 32 || block == 64 || block == 128 || block == 256; }
 inline int elem_bytes(int dtype) { return dtype == FR_FP8_E4M3 ? 1 : 2; }
@@ -68,14 +79,12 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       // faster for the down projection, but 6 % slower for the gate/up GEMM (short K, register-starved
       // epilogue: the hand-off K tiles spill; without the hand-off it is within 1 % of the plain kernel),
       // which keeps the plain kernel.
-      if constexpr (sizeof(T) == 1 && EPI == EPI_SILU) return launch_gemm<T, typename TL::T256, EPI>(a, splits, st);
+      if constexpr (sizeof(T) == 1 && EPI == EPI_SILU) return launch_gemm<T, typename TL::T256G, EPI>(a, splits, st);
       else {
-#ifdef FR_QUAD
+        // 2-byte operands, long K: the 16x16x32 MFMA form (see Tiles::T256S)
         if constexpr (sizeof(T) == 2) {
-          const int rc = launch_gemm_quad<T, EPI>(a, splits, st);
-          if (rc != 1) return rc;
+          if (a.K >= kSmallMfmaMinK) return launch_gemm_persistent<T, typename TL::T256S, EPI>(a, splits, st);
         }
-#endif
         return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
       }
     case 128:
@@ -122,6 +131,9 @@ int prepare_tiles() {
   GemmArgs a = {};
   a.setup_only = 1;
   int rc = launch_gemm_persistent<T, typename TL::T256, EPI>(a, 1, nullptr);
+  if constexpr (sizeof(T) == 2) {
+    if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T256S, EPI>(a, 1, nullptr);
+  }
   if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T128P, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm<T, typename TL::T128, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm<T, typename TL::T64, EPI>(a, 1, nullptr);
