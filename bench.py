@@ -53,10 +53,12 @@ def layer_bytes(M, H, F, E, topk, active, bw=2, ba=2):
 class Layer:
     """Device buffers + staged calls through the C ABI for one (shape, M)."""
 
-    def __init__(self, torch, N, shape, M, w1, w2, seed, fp8=None, dtype=None, x_scale=1.0):
+    def __init__(self, torch, N, shape, M, w1, w2, seed, fp8=None, dtype=None, x_scale=1.0, prepared=False):
         self.torch, self.N, self.M = torch, N, M
         self.tdtype = dtype or torch.bfloat16
         self.code = N.dtype_code(self.tdtype)
+        # prepared: the layout flags prepare_weights returned for w1, w2; they ride on the weight-taking calls' dtype
+        self.wcode = self.code | int(prepared or 0)
         self.fp8 = fp8  # (w1q, w1_scale, w2q, w2_scale) or None
         self.H, self.F, self.E, self.topk = shape["H"], shape["F"], shape["E"], shape["topk"]
         dev = "cuda"
@@ -101,7 +103,7 @@ class Layer:
                                              self.topk, 1, self.out.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream))
             return
         N.check(N.lib().fr_fused_moe(self.x.data_ptr(), self.w1.data_ptr(), self.w2.data_ptr(), self.logits.data_ptr(),
-                                     N.FR_F32, self.M, self.H, self.F, self.E, self.topk, 1, self.code,
+                                     N.FR_F32, self.M, self.H, self.F, self.E, self.topk, 1, self.wcode,
                                      self.out.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream))
 
     def staged(self, events=None):
@@ -132,13 +134,13 @@ class Layer:
             rec(4)
             return
         N.check(lib.fr_moe_gateup_silu(self.x.data_ptr(), self.w1.data_ptr(), self.sorted.data_ptr(), self.eids.data_ptr(),
-                                       self.npost.data_ptr(), self.M, self.H, self.F, self.E, self.topk, p.block, self.code,
+                                       self.npost.data_ptr(), self.M, self.H, self.F, self.E, self.topk, p.block, self.wcode,
                                        self.act.data_ptr(), self.tail.data_ptr() if self.tail is not None else None,
                                        self.stream))
         rec(3)
         N.check(lib.fr_moe_down_combine(self.act.data_ptr(), self.w2.data_ptr(), self.tw.data_ptr(), self.sorted.data_ptr(),
                                         self.eids.data_ptr(), self.npost.data_ptr(), self.M, self.H, self.F, self.E,
-                                        self.topk, p.block, p.split_k, self.code, self.partial.data_ptr(),
+                                        self.topk, p.block, p.split_k, self.wcode, self.partial.data_ptr(),
                                         self.out.data_ptr(), self.tail.data_ptr() if self.tail is not None else None,
                                         self.stream))
         rec(4)
@@ -199,8 +201,8 @@ def time_layer(torch, layer, steps, warmup, flush=False):
     return wall_ms, stage_us, quant
 
 
-def measure(torch, N, shape, M, w1, w2, steps, warmup, seed, fp8=None, flush=False, dtype=None, x_scale=1.0):
-    layer = Layer(torch, N, shape, M, w1, w2, seed, fp8, dtype=dtype, x_scale=x_scale)
+def measure(torch, N, shape, M, w1, w2, steps, warmup, seed, fp8=None, flush=False, dtype=None, x_scale=1.0, prepared=False):
+    layer = Layer(torch, N, shape, M, w1, w2, seed, fp8, dtype=dtype, x_scale=x_scale, prepared=prepared)
     if fp8:  # pad rows of act beyond npost are never written: keep them finite for the staged quantisation
         layer.act.zero_()
     wall_ms, stage_us, quant = time_layer(torch, layer, steps, warmup, flush)

@@ -6,7 +6,7 @@ include/fast_route_hip.h.  There is no CPU or eager fallback: every operator
 raises if the native library is missing.
 """
 from . import _native  # noqa: F401
-from .layers.fused_moe import fused_moe, fused_experts  # noqa: F401
+from .layers.fused_moe import fused_moe, fused_experts, prepare_weights  # noqa: F401
 from .layers.fp8 import fused_moe_fp8, prepare_weights_fp8, quantize_rows_e4m3  # noqa: F401
 from .ops.fused_moe import moe_align_block_size, invoke_fused_moe_kernel  # noqa: F401
 from .ops.stable_route import fused_route, topk_softmax  # noqa: F401
@@ -15,6 +15,7 @@ from .tuning import get_tunables, prepare, reset_tunables, set_tunables, tunable
 __all__ = [
     "fused_moe",
     "fused_experts",
+    "prepare_weights",
     "fused_moe_fp8",
     "prepare_weights_fp8",
     "quantize_rows_e4m3",

@@ -9,6 +9,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfast_route_hip.so")
 
 FR_F16, FR_BF16, FR_F32, FR_FP8_E4M3, FR_I32, FR_I64 = range(6)
+FR_W1_TILED, FR_W2_TILED, FR_W_TILED = 0x100, 0x200, 0x300  # OR-ed into a dtype argument: w1 / w2 / both are in the layout of fr_moe_prepare_weights
 
 _SHAPE_ERRORS = (-1, -2, -3, -4, -5)  # argument errors -> AssertionError like the reference's asserts
 
@@ -33,6 +34,7 @@ SIGNATURES = {
     "fr_moe_grouped_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                     c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fr_moe_prepare": (c_int, [c_int]),
+    "fr_moe_prepare_weights": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "fr_moe_set_tunables": (c_int, [ctypes.POINTER(FrMoeTunables)]),
     "fr_moe_get_tunables": (c_int, [ctypes.POINTER(FrMoeTunables)]),
     "fr_moe_get_plan": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, c_int, ctypes.POINTER(FrMoePlan)]),

@@ -96,6 +96,7 @@ extern "C" int fr_moe_get_tunables(fr_moe_tunables* t) {
 
 extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk, int dtype, fr_moe_plan* plan) {
   FR_REQUIRE(plan, FR_E_NULL, "fr_moe_get_plan: null plan");
+  dtype &= ~FR_W_TILED;  // the plan does not depend on the weight layout
   int rc = check_layer_shapes("fr_moe_get_plan", M, H, F, E, topk, dtype);
   if (rc != FR_OK) return rc;
   const int64_t n = M * topk;
@@ -200,7 +201,7 @@ extern "C" int fr_fused_experts(const void* x, const void* w1, const void* w2, c
   FR_REQUIRE(x && w1 && w2 && topk_weights && topk_ids && out, FR_E_NULL, "fr_fused_experts: null pointer");
   FR_REQUIRE(workspace && workspace_bytes >= p.workspace_bytes, FR_E_WORKSPACE, "fr_fused_experts: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)p.workspace_bytes);
   FR_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FR_E_ALIGN, "fr_fused_experts: workspace must be 256-byte aligned");
-  Carve c = carve(workspace, M, H, F, E, topk, dtype, p);
+  Carve c = carve(workspace, M, H, F, E, topk, dtype & ~FR_W_TILED, p);
   rc = fr_moe_align(topk_ids, FR_I32, M * topk, E, p.block, c.sorted, c.expert_ids, c.npost, c.align_ws, c.align_ws_bytes, stream);
   if (rc != FR_OK) return rc;
   rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, c.tail, stream);
@@ -218,10 +219,11 @@ extern "C" int fr_fused_moe(const void* x, const void* w1, const void* w2, const
   FR_REQUIRE(x && w1 && w2 && logits && out, FR_E_NULL, "fr_fused_moe: null pointer");
   FR_REQUIRE(workspace && workspace_bytes >= p.workspace_bytes, FR_E_WORKSPACE, "fr_fused_moe: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)p.workspace_bytes);
   FR_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, FR_E_ALIGN, "fr_fused_moe: workspace must be 256-byte aligned");
-  Carve c = carve(workspace, M, H, F, E, topk, dtype, p);
-  // a handful of tokens: the gate/up launch gates and sorts by itself
-  rc = gateup_rows_routed(x, w1, logits, logits_dtype, M, H, F, E, topk, renormalize, p.block, dtype, c.act, c.topk_w,
-                          c.topk_ids, c.sorted, c.expert_ids, c.npost, static_cast<hipStream_t>(stream));
+  Carve c = carve(workspace, M, H, F, E, topk, dtype & ~FR_W_TILED, p);
+  // a handful of tokens: the gate/up launch gates and sorts by itself (row-major weights only)
+  rc = (dtype & FR_W1_TILED) ? 1
+                            : gateup_rows_routed(x, w1, logits, logits_dtype, M, H, F, E, topk, renormalize, p.block, dtype, c.act, c.topk_w,
+                                                 c.topk_ids, c.sorted, c.expert_ids, c.npost, static_cast<hipStream_t>(stream));
   if (rc < 0) return rc;
   if (rc == 1) {
     rc = route_and_align(logits, logits_dtype, M, E, topk, renormalize, p.block, c, nullptr, H, stream);
@@ -240,6 +242,8 @@ extern "C" int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, con
   int rc = fr_moe_get_plan(M, H, F, E, topk, FR_FP8_E4M3, &p);
   if (rc != FR_OK) return rc;
   if (M == 0) return FR_OK;
+  const int w2_flag = x_dtype & FR_W2_TILED;
+  x_dtype &= ~FR_W_TILED;
   FR_REQUIRE(x_dtype == FR_BF16, FR_E_DTYPE, "fr_fused_moe_fp8: activations must be bf16 (dtype %d)", x_dtype);
   FR_REQUIRE(x && w1q && w1_scale && w2q && w2_scale && logits && out, FR_E_NULL, "fr_fused_moe_fp8: null pointer");
   FR_REQUIRE(workspace && workspace_bytes >= p.workspace_bytes, FR_E_WORKSPACE, "fr_fused_moe_fp8: workspace %lld < %lld bytes", (long long)workspace_bytes, (long long)p.workspace_bytes);
@@ -253,7 +257,7 @@ extern "C" int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, con
   rc = quant_rows(c.act, FR_BF16, p.sorted_len, c.npost, F, F, c.actq, c.act_scale, st);
   if (rc != FR_OK) return rc;
   return fr_moe_down_combine_fp8(c.actq, c.act_scale, w2q, w2_scale, c.topk_w, c.sorted, c.expert_ids, c.npost, M, H, F, E,
-                                 topk, p.block, p.split_k, x_dtype, c.partial, out, c.tail, stream);
+                                 topk, p.block, p.split_k, x_dtype | w2_flag, c.partial, out, c.tail, stream);
 }
 
 // ---- one entry point that allocates nothing ------------------------------------
@@ -292,7 +296,7 @@ extern "C" int fr_fused_moe_noalloc(const void* x, const void* w1, const void* w
   fr_moe_plan p;
   int rc = fr_moe_get_plan(M, H, F, E, topk, dtype, &p);
   if (rc != FR_OK) return rc;
-  FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "fr_fused_moe_noalloc: dtype %d not in {f16, bf16}", dtype);
+  FR_REQUIRE((dtype & ~FR_W_TILED) == FR_F16 || (dtype & ~FR_W_TILED) == FR_BF16, FR_E_DTYPE, "fr_fused_moe_noalloc: dtype %d not in {f16, bf16}", dtype);
   FR_REQUIRE(p.workspace_bytes <= kStaticScratchBytes, FR_E_WORKSPACE,
              "fr_fused_moe_noalloc: these sizes need %lld bytes of scratch, the library's static scratch holds %lld; use fr_fused_moe with a workspace",
              (long long)p.workspace_bytes, (long long)kStaticScratchBytes);

@@ -117,8 +117,10 @@ int64_t tail_scratch_bytes(int block, int dtype, int64_t K, int64_t N, bool gate
 int gateup_impl(const void* x, const float* x_scale, const void* w1, const float* w1_scale,
                 const int32_t* sorted, const int32_t* expert_ids, const int32_t* npost, int64_t M, int64_t H,
                 int64_t F, int E, int topk, int block, int dtype, void* act, float* tail_ws, hipStream_t st,
-                const char* who) {
+                const char* who, int w_tiled = 0) {
   if (M == 0) return FR_OK;
+  FR_REQUIRE(!w_tiled || (F % kTileRows == 0 && (H * elem_bytes(dtype)) % kTileBytes == 0), FR_E_SHAPE,
+             "%s: prepared weights need F %% %d == 0 and whole %d-byte K tiles", who, kTileRows, kTileBytes);
   FR_REQUIRE(x && w1 && act && sorted && expert_ids && npost, FR_E_NULL, "%s: null pointer", who);
   FR_REQUIRE(valid_block(block), FR_E_SHAPE, "%s: block=%d not in {16,32,64,128,256}", who, block);
   FR_REQUIRE(H > 0 && H % k_multiple(dtype, block) == 0, FR_E_SHAPE, "%s: H=%lld must be a multiple of %d for block %d", who, (long long)H, k_multiple(dtype, block), block);
@@ -133,10 +135,11 @@ int gateup_impl(const void* x, const float* x_scale, const void* w1, const float
   a.num_valid = (int)n; a.top_k = topk; a.N = (int)F; a.K = (int)H;
   a.num_experts = E;
   a.tail_ws = tail_ws;
+  a.w_tiled = w_tiled;
   // batches the routed form of the row kernel takes run the row kernel here too (same kernel, same sums, whoever
-  // did the routing)
+  // did the routing); the row kernels read whole weight rows and take the row-major layout only
   const int64_t min_k = gateup_rows_routes(M, E, topk, block) ? kRowsMinKRouted : kRowsMinK;
-  if (gateup_rows_fits(M, H, block, sorted_len, elem_bytes(dtype), min_k)) {
+  if (!w_tiled && gateup_rows_fits(M, H, block, sorted_len, elem_bytes(dtype), min_k)) {
     // a handful of tokens: stream the weight rows past the token rows without tiles
     if (dtype == FR_BF16) return launch_gateup_rows<bf16_t>(a, block, sorted_len / block * block, st);
     return launch_gateup_rows<f16_t>(a, block, sorted_len / block * block, st);
@@ -168,8 +171,10 @@ int gateup_rows_routed(const void* x, const void* w1, const void* logits, int lo
 int down_impl(const void* act, const float* act_scale, const void* w2, const float* w2_scale,
               const float* topk_weights, const int32_t* sorted, const int32_t* expert_ids, const int32_t* npost,
               int64_t M, int64_t H, int64_t F, int E, int topk, int block, int split_k, int dtype, int out_dtype,
-              float* partial, void* out, float* tail_ws, hipStream_t st, const char* who) {
+              float* partial, void* out, float* tail_ws, hipStream_t st, const char* who, int w_tiled = 0) {
   if (M == 0) return FR_OK;
+  FR_REQUIRE(!w_tiled || (H % kTileRows == 0 && (F * elem_bytes(dtype)) % kTileBytes == 0), FR_E_SHAPE,
+             "%s: prepared weights need H %% %d == 0 and whole %d-byte K tiles", who, kTileRows, kTileBytes);
   FR_REQUIRE(act && w2 && topk_weights && partial && out && sorted && expert_ids && npost, FR_E_NULL, "%s: null pointer", who);
   FR_REQUIRE(valid_block(block), FR_E_SHAPE, "%s: block=%d not in {16,32,64,128,256}", who, block);
   FR_REQUIRE(F > 0 && F % k_multiple(dtype, block) == 0, FR_E_SHAPE, "%s: F=%lld must be a multiple of %d for block %d", who, (long long)F, k_multiple(dtype, block), block);
@@ -189,7 +194,8 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
   a.num_experts = E;
   a.tail_ws = tail_ws;
   a.long_k = 1;
-  if (down_rows_fits(n, F, H, sorted_len, elem_bytes(dtype)) && out_dtype == dtype) {
+  a.w_tiled = w_tiled;
+  if (!w_tiled && down_rows_fits(n, F, H, sorted_len, elem_bytes(dtype)) && out_dtype == dtype) {
     // a handful of pairs: weight rows streamed past the activated rows, routed weight and top-k sum in the same kernel
     a.out = out;
     if (dtype == FR_BF16) return launch_down_rows<bf16_t>(a, topk, block, sorted_len, st);
@@ -206,15 +212,47 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
   return launch_combine(partial, FR_F32, n * H, splits, topk, M, (int)H, out_dtype, out, st);
 }
 
+// ---- prepared weight layout -----------------------------------------------------------------
+// One thread per 16-byte chunk of the OUTPUT (consecutive threads write consecutive memory): chunk o is
+// chunk c = o % 8 of row r = (o / 8) % 64 of K tile kt of row group g; its source is chunk kt * 8 + c of row
+// g * 64 + r of the row-major matrix (row groups never straddle experts: rows per expert are a multiple of 64).
+__global__ __launch_bounds__(256) void tile_weights_kernel(const u32x4* __restrict__ in, u32x4* __restrict__ out,
+                                                           int64_t chunks, int64_t ktiles) {
+  const int64_t o = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (o >= chunks) return;
+  constexpr int CPT = kTileBytes / 16;  // chunks per row and K tile
+  const int c = static_cast<int>(o % CPT), r = static_cast<int>((o / CPT) % kTileRows);
+  const int64_t piece = o / (CPT * kTileRows), kt = piece % ktiles, g = piece / ktiles;
+  out[o] = in[(g * kTileRows + r) * (ktiles * CPT) + kt * CPT + c];
+}
+
 }  // namespace fr
 
 using namespace fr;
+
+extern "C" int fr_moe_prepare_weights(const void* w, int dtype, int64_t E, int64_t rows, int64_t K, void* out, void* stream) {
+  FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16 || dtype == FR_FP8_E4M3, FR_E_DTYPE, "fr_moe_prepare_weights: dtype %d not in {f16, bf16, fp8_e4m3}", dtype);
+  FR_REQUIRE(w && out, FR_E_NULL, "fr_moe_prepare_weights: null pointer");
+  FR_REQUIRE(w != out, FR_E_SHAPE, "fr_moe_prepare_weights: not an in-place transform (out must not be w)");
+  const int es = elem_bytes(dtype);
+  FR_REQUIRE(E >= 1 && rows > 0 && rows % kTileRows == 0 && K > 0 && (K * es) % kTileBytes == 0, FR_E_SHAPE,
+             "fr_moe_prepare_weights: rows=%lld must be a multiple of %d and K=%lld a whole number of %d-byte tiles",
+             (long long)rows, kTileRows, (long long)K, kTileBytes);
+  FR_REQUIRE(aligned16(w) && aligned16(out), FR_E_ALIGN, "fr_moe_prepare_weights: operands must be 16-byte aligned");
+  const int64_t chunks = E * rows * K * es / 16;
+  FR_REQUIRE(ceil_div(chunks, 256) < (int64_t(1) << 31), FR_E_SHAPE, "fr_moe_prepare_weights: matrix too large");
+  hipLaunchKernelGGL(tile_weights_kernel, dim3(static_cast<unsigned>(ceil_div(chunks, 256))), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const u32x4*>(w), static_cast<u32x4*>(out), chunks, K * es / kTileBytes);
+  return check_launch("tile_weights_kernel");
+}
 
 extern "C" int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, void* C,
                                    const float* topk_weights, const int32_t* sorted_token_ids,
                                    const int32_t* expert_ids, const int32_t* num_tokens_post_pad,
                                    int64_t sorted_len, int64_t num_valid, int64_t N, int64_t K, int E,
                                    int block, int top_k, int mul_routed_weight, int dtype, void* stream) {
+  const int w_tiled = (dtype & FR_W_TILED) ? 1 : 0;
+  dtype &= ~FR_W_TILED;
   if (num_valid == 0) return FR_OK;
   FR_REQUIRE(A && B && C && sorted_token_ids && expert_ids && num_tokens_post_pad, FR_E_NULL, "fr_moe_grouped_gemm: null pointer");
   FR_REQUIRE(!mul_routed_weight || topk_weights, FR_E_NULL, "fr_moe_grouped_gemm: mul_routed_weight without topk_weights");
@@ -231,6 +269,8 @@ extern "C" int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, vo
   a.topk_w = topk_weights; a.num_valid = (int)num_valid; a.top_k = top_k; a.N = (int)N; a.K = (int)K;
   a.mul_weight = mul_routed_weight;
   a.num_experts = E;
+  FR_REQUIRE(!w_tiled || (N % kTileRows == 0 && (K * 2) % kTileBytes == 0), FR_E_SHAPE, "fr_moe_grouped_gemm: prepared weights need N %% %d == 0", kTileRows);
+  a.w_tiled = w_tiled;
   // only whole blocks inside sorted_token_ids are addressable
   return dispatch_dtype<EPI_PLAIN>(a, dtype, block, 1, sorted_len / block * block, static_cast<hipStream_t>(stream));
 }
@@ -239,9 +279,11 @@ extern "C" int fr_moe_gateup_silu(const void* x, const void* w1, const int32_t* 
                                   const int32_t* expert_ids, const int32_t* num_tokens_post_pad,
                                   int64_t M, int64_t H, int64_t F, int E, int topk, int block, int dtype,
                                   void* act, void* tail_ws, void* stream) {
+  const int w_tiled = (dtype & FR_W1_TILED) ? 1 : 0;
+  dtype &= ~FR_W_TILED;
   FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "fr_moe_gateup_silu: dtype %d not in {f16, bf16}", dtype);
   return gateup_impl(x, nullptr, w1, nullptr, sorted_token_ids, expert_ids, num_tokens_post_pad, M, H, F, E, topk,
-                     block, dtype, act, static_cast<float*>(tail_ws), static_cast<hipStream_t>(stream), "fr_moe_gateup_silu");
+                     block, dtype, act, static_cast<float*>(tail_ws), static_cast<hipStream_t>(stream), "fr_moe_gateup_silu", w_tiled);
 }
 
 extern "C" int fr_moe_gateup_silu_fp8(const void* xq, const float* x_scale, const void* w1q, const float* w1_scale,
@@ -258,10 +300,12 @@ extern "C" int fr_moe_down_combine(const void* act, const void* w2, const float*
                                    const int32_t* num_tokens_post_pad, int64_t M, int64_t H, int64_t F,
                                    int E, int topk, int block, int split_k, int dtype, float* partial,
                                    void* out, void* tail_ws, void* stream) {
+  const int w_tiled = (dtype & FR_W2_TILED) ? 1 : 0;
+  dtype &= ~FR_W_TILED;
   FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "fr_moe_down_combine: dtype %d not in {f16, bf16}", dtype);
   return down_impl(act, nullptr, w2, nullptr, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, M, H, F,
                    E, topk, block, split_k, dtype, dtype, partial, out, static_cast<float*>(tail_ws),
-                   static_cast<hipStream_t>(stream), "fr_moe_down_combine");
+                   static_cast<hipStream_t>(stream), "fr_moe_down_combine", w_tiled);
 }
 
 extern "C" int fr_moe_down_combine_fp8(const void* actq, const float* act_scale, const void* w2q, const float* w2_scale,
@@ -269,10 +313,12 @@ extern "C" int fr_moe_down_combine_fp8(const void* actq, const float* act_scale,
                                        const int32_t* expert_ids, const int32_t* num_tokens_post_pad, int64_t M,
                                        int64_t H, int64_t F, int E, int topk, int block, int split_k, int out_dtype,
                                        float* partial, void* out, void* tail_ws, void* stream) {
+  const int w_tiled = (out_dtype & FR_W2_TILED) ? 1 : 0;
+  out_dtype &= ~FR_W_TILED;
   FR_REQUIRE(act_scale && w2_scale, FR_E_NULL, "fr_moe_down_combine_fp8: null scale pointer");
   return down_impl(actq, act_scale, w2q, w2_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, M,
                    H, F, E, topk, block, split_k, FR_FP8_E4M3, out_dtype, partial, out, static_cast<float*>(tail_ws),
-                   static_cast<hipStream_t>(stream), "fr_moe_down_combine_fp8");
+                   static_cast<hipStream_t>(stream), "fr_moe_down_combine_fp8", w_tiled);
 }
 
 // Every kernel the grouped GEMM entry points can launch for `dtype`, set up on the current device.

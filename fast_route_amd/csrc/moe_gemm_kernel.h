@@ -60,10 +60,25 @@ struct GemmArgs {
   int num_experts;      // E (persistent form: walk order by expert)
   int long_k;           // down projection (few feature tiles, long K): hint for the 128-row tile's form
   float* tail_ws;       // persistent form only: slice buffers for splitting the last round of tiles along K, or nullptr
+  int w_tiled;          // W is in the prepared layout (see w_byte_offset), not [E, w_rows, K] row-major
   int setup_only;       // do the per-device set-up of the kernel a launch would take (LDS limit, occupancy) and launch nothing
 };
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Prepared weight layout (fr_moe_prepare_weights): inside an expert, groups of kTileRows consecutive rows; inside a
+// group, K tiles of kTileBytes per row; inside a K tile the group's rows one after the other.  A (row group, K tile)
+// piece is 8 KB of consecutive memory, a group's whole K range one run of memory, where the row-major layout has a
+// weight tile in as many 128-byte pieces as it has rows, one row length apart.
+constexpr int kTileRows = 64, kTileBytes = 128, kTilePiece = kTileRows * kTileBytes;
+// byte offset of byte kb of row `row` inside one expert's weights; es = bytes per element
+__device__ __host__ __forceinline__ int64_t w_byte_offset(int w_tiled, int64_t ldw, int64_t K, int row, int64_t kb, int es) {
+  if (w_tiled) {
+    const int64_t ktiles = (K * es) / kTileBytes;
+    return ((static_cast<int64_t>(row / kTileRows) * ktiles + kb / kTileBytes) * kTilePiece) + (row % kTileRows) * kTileBytes + kb % kTileBytes;
+  }
+  return static_cast<int64_t>(row) * ldw * es + kb;
+}
 struct fp8_t { unsigned char bits; };  // OCP e4m3fn storage
 
 // Element traits: FC = 16-byte chunks one lane feeds to one MFMA, out_t = type the
@@ -520,6 +535,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     const __amdgpu_buffer_rsrc_t xrs = uniform_rsrc(X + xrow0 * a.ldx);
     const __amdgpu_buffer_rsrc_t wrs = uniform_rsrc(W);
     const bool issuer = wave_u < NW / IW;
+    const int wstep = a.w_tiled ? (C::BKB / kTileBytes) * kTilePiece : C::BKB;  // bytes from one K tile of W to the next
     unsigned xsrc[XI * IW], wsrc[WI * IW];  // byte offsets, [load][virtual wavefront]
 #pragma unroll
     for (int ih = 0; ih < XI * IW; ++ih) {
@@ -533,7 +549,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
       const int i = ih / IW, vw = (wave_u + (ih % IW) * (NW / IW)) % NW;
       const int slot = (i * NW + vw) * kWave + lane;
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
-      wsrc[ih] = static_cast<unsigned>((static_cast<int64_t>(w_src_row(rr)) * a.ldw + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));
+      wsrc[ih] = static_cast<unsigned>(w_byte_offset(a.w_tiled, a.ldw, a.K, w_src_row(rr), (k0 + c * EPC) * static_cast<int64_t>(sizeof(T)), sizeof(T)));
     }
     // load q_ of an issuing wavefront of tile tile_ into ring slot slot_.  Weight-tile loads come
     // first: in the prologue they depend only on the expert id, so they are in flight while the
@@ -545,7 +561,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     if ((q_) < WI * IW) {                                                                                  \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
           wrs, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vw_) * (kWave * 16)), \
-          16, wsrc[(q_) < WI * IW ? (q_) : 0], (tile_) * C::BKB, 0, FR_W_AUX);                                    \
+          16, wsrc[(q_) < WI * IW ? (q_) : 0], (tile_) * wstep, 0, FR_W_AUX);                                    \
     } else {                                                                                               \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
           xrs, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WI * IW) / IW) * NW + vw_) * (kWave * 16)), \
@@ -682,6 +698,7 @@ int launch_gemm(const GemmArgs& a, int splits, hipStream_t st) {
     }
   }
   if (a.setup_only) return FR_OK;
+  if (C::STAGES == 0 && a.w_tiled) return fail(FR_E_SHAPE, "prepared weights need a direct-to-LDS tile");
   if (C::STAGES > 0) {  // the ring loads address rows by 32-bit byte offsets
     const int64_t x_rows = a.top_k > 0 ? a.num_valid / a.top_k : C::BT;
     const int64_t w_rows = EPI == EPI_SILU ? 2 * static_cast<int64_t>(a.N) : a.N;

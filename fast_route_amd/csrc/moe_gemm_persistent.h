@@ -199,6 +199,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   const int wt = wave / C::WF, wf = wave % C::WF;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const bool issuer = wave_u < NW / IW;
+  const int wstep = a.w_tiled ? (C::BKB / kTileBytes) * kTilePiece : C::BKB;  // bytes from one K tile of W to the next
   const T* X = static_cast<const T*>(a.X);
 
   // unit j_ -> tile coordinates, first K tile kb_ and K tile count kn_, slice buffer tu_ (-1: a whole tile)
@@ -269,8 +270,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     }                                                                                                        \
     _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) {                                                 \
       FR_SLOT_ROW(ih, rr, c)                                                                                 \
-      wsrc_[ih] = static_cast<unsigned>((static_cast<int64_t>(w_src_row(pf_, rr)) * a.ldw + kfirst_ + c * EPC) * \
-                                        static_cast<int64_t>(sizeof(T)));                                    \
+      wsrc_[ih] = static_cast<unsigned>(w_byte_offset(a.w_tiled, a.ldw, a.K, w_src_row(pf_, rr),             \
+                                                      (kfirst_ + c * EPC) * static_cast<int64_t>(sizeof(T)), sizeof(T))); \
     }                                                                                                        \
   }
   FR_UNIT(0, pid_t, pid_f, expert, kb, kn, tu)
@@ -287,8 +288,10 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   // load q_ of an issuing wavefront (weight-tile loads first) of K tile tile_ into ring slot slot_
 #ifdef FR_ABL_HOTLOAD
 #define FR_KOFF(tile_) (((tile_) & 3) * C::BKB)
+#define FR_KOFF_W(tile_) (((tile_) & 3) * wstep)
 #else
 #define FR_KOFF(tile_) ((tile_) * C::BKB)
+#define FR_KOFF_W(tile_) ((tile_) * wstep)
 #endif
 #define FR_ISSUE_REAL(SET, tile_, slot_, q_)                                                                \
   {                                                                                                         \
@@ -296,7 +299,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     if ((q_) < WI * IW) {                                                                                   \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
           wrs##SET, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vwi_) * (kWave * 16)), \
-          16, wsrc##SET[(q_) < WI * IW ? (q_) : 0], FR_KOFF(tile_), 0, 0);                                      \
+          16, wsrc##SET[(q_) < WI * IW ? (q_) : 0], FR_KOFF_W(tile_), 0, 0);                                      \
     } else {                                                                                                \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
           xrs##SET, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WI * IW) / IW) * NW + vwi_) * (kWave * 16)), \
@@ -519,6 +522,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #undef FR_READ_FRAGS_REAL
 #undef FR_ABL_INIT1
 #undef FR_KOFF
+#undef FR_KOFF_W
 #undef FR_MFMA
 #undef FR_KT_BARRIER
 #undef FR_MAKE_SET

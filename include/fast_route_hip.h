@@ -94,6 +94,37 @@ int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, void* C,
                         int64_t sorted_len, int64_t num_valid, int64_t N, int64_t K, int E,
                         int block, int top_k, int mul_routed_weight, int dtype, void* stream);
 
+/* ---- prepared weight layout (optional) -------------------------------------
+ * The reference takes w1 [E, 2F, H] and w2 [E, H, F] row-major
+ * (fast_route/fast_route/layers/stable_route.py:32-36; gate rows first, up rows second,
+ * fast_route/benchmarks/fused_route/activation.py:27-30) and so does every entry point here.
+ * A weight tile of a GEMM is then as many 128-byte pieces as it has rows, one row length
+ * apart.  fr_moe_prepare_weights re-lays a weight matrix w[E, rows, K] out once, into a
+ * buffer `out` of the same size (the caller may free `w` afterwards; not in place):
+ * inside an expert, groups of 64 consecutive rows; inside a group, K tiles of 128 bytes per
+ * row; inside a K tile the group's 64 rows one after the other - each (row group, K tile)
+ * is 8 KB of consecutive memory and a group's whole K range one run.
+ * rows % 64 == 0, K * element size % 128 == 0; dtype in {FR_F16, FR_BF16, FR_FP8_E4M3}.
+ * Entry points that take a `dtype` argument accept layout flags OR-ed into it: FR_W1_TILED - the
+ * gate/up weights (w1; B of fr_moe_grouped_gemm) are in this layout -, FR_W2_TILED - the down
+ * weights (w2) are -, FR_W_TILED = both.  fr_moe_gateup_silu looks at FR_W1_TILED,
+ * fr_moe_down_combine at FR_W2_TILED, fr_moe_grouped_gemm at either, fr_fused_experts,
+ * fr_fused_moe and fr_fused_moe_noalloc at both; the fp8 entry points take the flags in
+ * their `out_dtype` (fr_moe_down_combine_fp8: FR_W2_TILED) and `x_dtype` (fr_fused_moe_fp8:
+ * FR_W2_TILED) arguments, for codes tiled with dtype FR_FP8_E4M3 (128 elements per K tile).
+ * Results are bit-identical to the row-major call when the same kernels run; with FR_W1_TILED
+ * (FR_W2_TILED) batches of up to 4 tokens (4 pairs), whose row-major form streams whole weight
+ * rows without tiles, take the 16-row tile kernels instead.
+ * Measured on the Mixtral shape: the down projection is 2-7 % faster from 512 tokens up and
+ * never slower; the gate/up GEMM gains under 1 % from 512 tokens up and loses 2-6 % below
+ * (its decode tiles stream 512-byte pieces of the 8 KB weight rows) - prepare w2 always,
+ * w1 only for a prefill-only deployment. */
+#define FR_W1_TILED 0x100
+#define FR_W2_TILED 0x200
+#define FR_W_TILED 0x300
+int fr_moe_prepare_weights(const void* w, int dtype, int64_t E, int64_t rows, int64_t K, void* out,
+                           void* stream);
+
 /* ---- fused expert MLPs ---------------------------------------------------
  * Tile plan chosen from the problem size: the routing block the fused kernels
  * want (pass it to fr_moe_align) and the split-K factor of the down GEMM. */

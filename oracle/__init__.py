@@ -19,6 +19,7 @@ from .moe_oracle import (  # noqa: F401
     quant_e4m3_rows,
     quantize_weights_fp8,
     fused_moe_fp8,
+    tile_weights,
     make_inputs,
     zipf_logits,
 )

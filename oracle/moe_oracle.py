@@ -299,6 +299,20 @@ def fused_moe_fp8(hidden_states, w1, w2, gating_output, topk: int, renormalize: 
 
 
 # --------------------------------------------------------------------------
+# prepared weight layout (no counterpart in the reference, which keeps w1 [E, 2F, H] / w2 [E, H, F]
+# row-major: layers/stable_route.py:32-36): a pure permutation of the elements, restated with a reshape
+# --------------------------------------------------------------------------
+def tile_weights(w: torch.Tensor, rows_per_group: int = 64, tile_bytes: int = 128) -> torch.Tensor:
+    """w [E, rows, K] -> same shape holding [E][rows/64][K tiles][64 rows][tile_bytes / itemsize] flat.
+    Pinned in tests/test_oracle.py by an element-by-element loop over the definition."""
+    E, rows, K = w.shape
+    el = tile_bytes // w.element_size()
+    assert rows % rows_per_group == 0 and K % el == 0
+    t = w.reshape(E, rows // rows_per_group, rows_per_group, K // el, el).permute(0, 1, 3, 2, 4)
+    return t.contiguous().reshape(E, rows, K)
+
+
+# --------------------------------------------------------------------------
 # seeded synthetic inputs (shared by tests, smoke and bench)
 # --------------------------------------------------------------------------
 def zipf_logits(M: int, E: int, seed: int, s: float = 1.2, tau: float = 1.0) -> torch.Tensor:

@@ -362,3 +362,23 @@ def test_fp8_layer_oracle_against_independent_per_pair_loop():
         assert (got - want).abs().max() <= tol, (got - want).abs().max()
         for mistake in ("per_tensor_scale", "no_bf16_rounding", "no_requantisation"):
             assert (got - layer(x, logits, w1, w2, k, mistake)).abs().max() > 20 * tol, mistake
+
+
+def test_tile_weights_is_the_stated_permutation():
+    """oracle.tile_weights against the layout's definition, element by element: element (e, row, k) lands at flat
+    offset ((row // 64) * ktiles + k // el) * 64 * el + (row % 64) * el + k % el of expert e."""
+    import oracle
+    torch.manual_seed(5)
+    for dtype, el in ((torch.bfloat16, 64), (torch.uint8, 128)):
+        E, rows, K = 2, 128, 2 * el
+        w = torch.arange(E * rows * K, dtype=torch.int32).reshape(E, rows, K) % 251
+        w = w.to(dtype)
+        t = oracle.tile_weights(w).reshape(E, -1)
+        ktiles = K // el
+        for e in range(E):
+            for row in (0, 1, 63, 64, 65, 127):
+                for k in (0, 1, el - 1, el, K - 1):
+                    off = ((row // 64) * ktiles + k // el) * 64 * el + (row % 64) * el + k % el
+                    assert t[e, off] == w[e, row, k], (e, row, k)
+        # a permutation: nothing lost, nothing duplicated
+        assert torch.equal(torch.sort(t.flatten().int())[0], torch.sort(w.flatten().int())[0])
