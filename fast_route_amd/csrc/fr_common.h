@@ -38,6 +38,15 @@ int gateup_rows_routed(const void* x, const void* w1, const void* logits, int lo
                        int64_t F, int E, int topk, int renorm, int block, int dtype, void* act, float* topk_w,
                        int32_t* topk_ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, hipStream_t st);
 
+// Down projection + routed weight + top-k combine (what fr_moe_down_combine / fr_moe_down_combine_fp8 launch).  pair_ids:
+// the [M, topk] expert ids, or nullptr; with them a pair whose id lies outside [0, E) - it has no slot in the routing
+// arrays - contributes nothing to its token's sum (without them its never-written partial row would be added).
+int down_impl(const void* act, const float* act_scale, const void* w2, const float* w2_scale,
+              const float* topk_weights, const int32_t* sorted, const int32_t* expert_ids, const int32_t* npost,
+              int64_t M, int64_t H, int64_t F, int E, int topk, int block, int split_k, int dtype, int out_dtype,
+              float* partial, void* out, float* tail_ws, hipStream_t st, const char* who, int w_tiled,
+              const int32_t* pair_ids);
+
 #define FR_REQUIRE(cond, code, ...) \
   do {                              \
     if (!(cond)) return ::fr::fail((code), __VA_ARGS__); \

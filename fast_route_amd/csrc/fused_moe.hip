@@ -206,7 +206,9 @@ extern "C" int fr_fused_experts(const void* x, const void* w1, const void* w2, c
   if (rc != FR_OK) return rc;
   rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, c.tail, stream);
   if (rc != FR_OK) return rc;
-  return fr_moe_down_combine(c.act, w2, topk_weights, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, p.split_k, dtype, c.partial, out, c.tail, stream);
+  return down_impl(c.act, nullptr, w2, nullptr, topk_weights, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block,
+                   p.split_k, dtype & ~FR_W_TILED, dtype & ~FR_W_TILED, c.partial, out, c.tail, static_cast<hipStream_t>(stream),
+                   "fr_fused_experts", (dtype & FR_W2_TILED) ? 1 : 0, topk_ids);
 }
 
 extern "C" int fr_fused_moe(const void* x, const void* w1, const void* w2, const void* logits, int logits_dtype,
@@ -231,7 +233,9 @@ extern "C" int fr_fused_moe(const void* x, const void* w1, const void* w2, const
     rc = fr_moe_gateup_silu(x, w1, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, dtype, c.act, c.tail, stream);
     if (rc != FR_OK) return rc;
   }
-  return fr_moe_down_combine(c.act, w2, c.topk_w, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block, p.split_k, dtype, c.partial, out, c.tail, stream);
+  return down_impl(c.act, nullptr, w2, nullptr, c.topk_w, c.sorted, c.expert_ids, c.npost, M, H, F, E, topk, p.block,
+                   p.split_k, dtype & ~FR_W_TILED, dtype & ~FR_W_TILED, c.partial, out, c.tail, static_cast<hipStream_t>(stream),
+                   "fr_fused_moe", (dtype & FR_W2_TILED) ? 1 : 0, c.topk_ids);
 }
 
 extern "C" int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, const float* w1_scale, const void* w2q,

@@ -11,7 +11,8 @@ namespace fr {
 template <typename T, typename P, int V>
 __global__ __launch_bounds__(256) void combine_kernel(const P* __restrict__ partial,
                                                       int64_t split_stride, int splits, int topk,
-                                                      int64_t M, int H, T* __restrict__ out) {
+                                                      int64_t M, int H, T* __restrict__ out,
+                                                      const int32_t* __restrict__ pair_ids, int E) {
   typedef P pv __attribute__((ext_vector_type(V)));
   typedef T tv __attribute__((ext_vector_type(V)));
   const int64_t idx = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * V;
@@ -21,12 +22,17 @@ __global__ __launch_bounds__(256) void combine_kernel(const P* __restrict__ part
   float s[V];
 #pragma unroll
   for (int r = 0; r < V; ++r) s[r] = 0.f;
-  for (int j = 0; j < topk; ++j)
+  for (int j = 0; j < topk; ++j) {
+    if (pair_ids) {  // a pair whose expert id lies outside [0, E) got no slot in the routing arrays: no row was written for it
+      const int e = pair_ids[m * topk + j];
+      if (e < 0 || e >= E) continue;
+    }
     for (int sp = 0; sp < splits; ++sp) {
       const pv v = *reinterpret_cast<const pv*>(partial + sp * split_stride + (m * topk + j) * H + h);
 #pragma unroll
       for (int r = 0; r < V; ++r) s[r] += static_cast<float>(v[r]);
     }
+  }
   tv o;
 #pragma unroll
   for (int r = 0; r < V; ++r) o[r] = static_cast<T>(s[r]);
@@ -59,38 +65,43 @@ int dispatch_dtype(const GemmArgs& a, int dtype, int block, int splits, int64_t 
 
 template <typename T, typename P>
 void launch_combine_as(const void* partial, int64_t split_stride, int splits, int topk, int64_t M, int H, void* out,
-                       hipStream_t st) {
+                       const int32_t* pair_ids, int E, hipStream_t st) {
   // 16-byte loads of the 2-byte rows of a single slice when the row length allows, else 4 elements per thread
   if (sizeof(P) == 2 && H % 8 == 0) {
     const unsigned grid = static_cast<unsigned>(ceil_div(M * H / 8, 256));
     hipLaunchKernelGGL((combine_kernel<T, P, 8>), dim3(grid), dim3(256), 0, st, static_cast<const P*>(partial), split_stride,
-                       splits, topk, M, H, static_cast<T*>(out));
+                       splits, topk, M, H, static_cast<T*>(out), pair_ids, E);
     return;
   }
   const unsigned grid = static_cast<unsigned>(ceil_div(M * H / 4, 256));
   hipLaunchKernelGGL((combine_kernel<T, P, 4>), dim3(grid), dim3(256), 0, st, static_cast<const P*>(partial), split_stride,
-                     splits, topk, M, H, static_cast<T*>(out));
+                     splits, topk, M, H, static_cast<T*>(out), pair_ids, E);
 }
 
 // partial_dtype: FR_F32, or the 2-byte type a single slice was written in
 int launch_combine(const void* partial, int partial_dtype, int64_t split_stride, int splits, int topk, int64_t M, int H,
-                   int out_dtype, void* out, hipStream_t st) {
+                   int out_dtype, void* out, const int32_t* pair_ids, int E, hipStream_t st) {
   if (M == 0) return FR_OK;
   if (out_dtype != FR_BF16 && out_dtype != FR_F16) return fail(FR_E_DTYPE, "output dtype %d not in {f16, bf16}", out_dtype);
   const bool ob = out_dtype == FR_BF16;
   if (partial_dtype == FR_F32) {
-    if (ob) launch_combine_as<bf16_t, float>(partial, split_stride, splits, topk, M, H, out, st);
-    else launch_combine_as<f16_t, float>(partial, split_stride, splits, topk, M, H, out, st);
+    if (ob) launch_combine_as<bf16_t, float>(partial, split_stride, splits, topk, M, H, out, pair_ids, E, st);
+    else launch_combine_as<f16_t, float>(partial, split_stride, splits, topk, M, H, out, pair_ids, E, st);
   } else if (partial_dtype == FR_BF16) {
-    if (ob) launch_combine_as<bf16_t, bf16_t>(partial, split_stride, splits, topk, M, H, out, st);
-    else launch_combine_as<f16_t, bf16_t>(partial, split_stride, splits, topk, M, H, out, st);
+    if (ob) launch_combine_as<bf16_t, bf16_t>(partial, split_stride, splits, topk, M, H, out, pair_ids, E, st);
+    else launch_combine_as<f16_t, bf16_t>(partial, split_stride, splits, topk, M, H, out, pair_ids, E, st);
   } else if (partial_dtype == FR_F16) {
-    if (ob) launch_combine_as<bf16_t, f16_t>(partial, split_stride, splits, topk, M, H, out, st);
-    else launch_combine_as<f16_t, f16_t>(partial, split_stride, splits, topk, M, H, out, st);
+    if (ob) launch_combine_as<bf16_t, f16_t>(partial, split_stride, splits, topk, M, H, out, pair_ids, E, st);
+    else launch_combine_as<f16_t, f16_t>(partial, split_stride, splits, topk, M, H, out, pair_ids, E, st);
   } else {
     return fail(FR_E_DTYPE, "partial dtype %d", partial_dtype);
   }
   return check_launch("combine_kernel");
+}
+
+__global__ __launch_bounds__(256) void zero_fill_kernel(u32x4* __restrict__ p, int64_t n16) {
+  const u32x4 z = {0u, 0u, 0u, 0u};
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n16; i += static_cast<int64_t>(gridDim.x) * 256) p[i] = z;
 }
 
 // a split whose K range is empty would leave its slice unwritten: shrink until every slice has work
@@ -171,7 +182,8 @@ int gateup_rows_routed(const void* x, const void* w1, const void* logits, int lo
 int down_impl(const void* act, const float* act_scale, const void* w2, const float* w2_scale,
               const float* topk_weights, const int32_t* sorted, const int32_t* expert_ids, const int32_t* npost,
               int64_t M, int64_t H, int64_t F, int E, int topk, int block, int split_k, int dtype, int out_dtype,
-              float* partial, void* out, float* tail_ws, hipStream_t st, const char* who, int w_tiled = 0) {
+              float* partial, void* out, float* tail_ws, hipStream_t st, const char* who, int w_tiled,
+              const int32_t* pair_ids) {
   if (M == 0) return FR_OK;
   FR_REQUIRE(!w_tiled || (H % kTileRows == 0 && (F * elem_bytes(dtype)) % kTileBytes == 0), FR_E_SHAPE,
              "%s: prepared weights need H %% %d == 0 and whole %d-byte K tiles", who, kTileRows, kTileBytes);
@@ -202,14 +214,32 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
     return launch_down_rows<f16_t>(a, topk, block, sorted_len, st);
   }
   if (splits == 1) {
+    const int row_dtype = dtype == FR_F16 ? FR_F16 : FR_BF16;  // type a single slice's rows are written in
+    if (topk == 2 && out_dtype == row_dtype) {
+      // Two pairs per token: the combine happens in the GEMM epilogue.  `out` is zero-filled (by a kernel: the call
+      // stays capturable) and every pair's weighted row is added into its token's row with packed atomics - 0 + a
+      // is exact and a + b is rounded once, so the result does not depend on which pair arrives first and equals
+      // the sum the combine kernel would form from the same two rounded rows.  No partial rows, no combine launch;
+      // a pair whose expert id is out of range has no slot and adds nothing.
+      const int64_t n16 = M * H * 2 / 16;  // H % 4 == 0 and 16-byte alignment were checked; M * H * 2 % 16: see below
+      if ((M * H) % 8 == 0) {
+        hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>(ceil_div(n16, 256) < 4096 ? ceil_div(n16, 256) : 4096)),
+                           dim3(256), 0, st, static_cast<u32x4*>(out), n16);
+        int rc = check_launch("zero_fill_kernel");
+        if (rc != FR_OK) return rc;
+        a.out = out;
+        a.add_div = topk;
+        return dispatch_dtype<EPI_PLAIN>(a, dtype, block, 1, sorted_len / block * block, st);
+      }
+    }
     // one slice: each pair's row in the operands' 2-byte type (bf16 for fp8 operands), half the partial traffic
     int rc = dispatch_dtype<EPI_PLAIN>(a, dtype, block, 1, sorted_len / block * block, st);
     if (rc != FR_OK) return rc;
-    return launch_combine(partial, dtype == FR_F16 ? FR_F16 : FR_BF16, n * H, 1, topk, M, (int)H, out_dtype, out, st);
+    return launch_combine(partial, row_dtype, n * H, 1, topk, M, (int)H, out_dtype, out, pair_ids, E, st);
   }
   int rc = dispatch_dtype<EPI_DOWN>(a, dtype, block, splits, sorted_len / block * block, st);
   if (rc != FR_OK) return rc;
-  return launch_combine(partial, FR_F32, n * H, splits, topk, M, (int)H, out_dtype, out, st);
+  return launch_combine(partial, FR_F32, n * H, splits, topk, M, (int)H, out_dtype, out, pair_ids, E, st);
 }
 
 // ---- prepared weight layout -----------------------------------------------------------------
@@ -305,7 +335,7 @@ extern "C" int fr_moe_down_combine(const void* act, const void* w2, const float*
   FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "fr_moe_down_combine: dtype %d not in {f16, bf16}", dtype);
   return down_impl(act, nullptr, w2, nullptr, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, M, H, F,
                    E, topk, block, split_k, dtype, dtype, partial, out, static_cast<float*>(tail_ws),
-                   static_cast<hipStream_t>(stream), "fr_moe_down_combine", w_tiled);
+                   static_cast<hipStream_t>(stream), "fr_moe_down_combine", w_tiled, nullptr);
 }
 
 extern "C" int fr_moe_down_combine_fp8(const void* actq, const float* act_scale, const void* w2q, const float* w2_scale,
@@ -318,7 +348,7 @@ extern "C" int fr_moe_down_combine_fp8(const void* actq, const float* act_scale,
   FR_REQUIRE(act_scale && w2_scale, FR_E_NULL, "fr_moe_down_combine_fp8: null scale pointer");
   return down_impl(actq, act_scale, w2q, w2_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_pad, M,
                    H, F, E, topk, block, split_k, FR_FP8_E4M3, out_dtype, partial, out, static_cast<float*>(tail_ws),
-                   static_cast<hipStream_t>(stream), "fr_moe_down_combine_fp8", w_tiled);
+                   static_cast<hipStream_t>(stream), "fr_moe_down_combine_fp8", w_tiled, nullptr);
 }
 
 // Every kernel the grouped GEMM entry points can launch for `dtype`, set up on the current device.

@@ -60,6 +60,7 @@ struct GemmArgs {
   int num_experts;      // E (persistent form: walk order by expert)
   int long_k;           // down projection (few feature tiles, long K): hint for the 128-row tile's form
   float* tail_ws;       // persistent form only: slice buffers for splitting the last round of tiles along K, or nullptr
+  int add_div;          // EPI_PLAIN: 0 = store row `sorted id` of out; k > 0 = add into row (sorted id / k) of a zero-filled out (packed atomics)
   int w_tiled;          // W is in the prepared layout (see w_byte_offset), not [E, w_rows, K] row-major
   int setup_only;       // do the per-device set-up of the kernel a launch would take (LDS limit, occupancy) and launch nothing
 };
@@ -127,6 +128,29 @@ template <> struct Elem<fp8_t> {
 
 // g * sigmoid(g).  The quotient is a multiplication by v_rcp_f32 (1 ulp) instead of the IEEE division's ten
 // instructions: the result is rounded to 8 or 11 bits right after, and the epilogue's VALU time is MFMA idle time.
+// out[0..3] += v (2-byte elements), two packed atomic adds.  With exactly two contributions to a zero-filled
+// element the result does not depend on their order: 0 + a is exact, a + b is rounded once.
+#if defined(__HIP_DEVICE_COMPILE__)
+__device__ __forceinline__ void atomic_add4(bf16_t* p, bf16x4 v) {
+  typedef short s2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  typedef __attribute__((address_space(1))) s2* gptr;
+  const b2 lo = {v[0], v[1]}, hi = {v[2], v[3]};
+  __builtin_amdgcn_global_atomic_fadd_v2bf16((gptr)(p), __builtin_bit_cast(s2, lo));
+  __builtin_amdgcn_global_atomic_fadd_v2bf16((gptr)(p + 2), __builtin_bit_cast(s2, hi));
+}
+__device__ __forceinline__ void atomic_add4(f16_t* p, f16x4 v) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  typedef __attribute__((address_space(1))) h2* gptr;
+  const h2 lo = {v[0], v[1]}, hi = {v[2], v[3]};
+  __builtin_amdgcn_global_atomic_fadd_v2f16((gptr)(p), lo);
+  __builtin_amdgcn_global_atomic_fadd_v2f16((gptr)(p + 2), hi);
+}
+#else
+__device__ __forceinline__ void atomic_add4(bf16_t*, bf16x4) {}
+__device__ __forceinline__ void atomic_add4(f16_t*, f16x4) {}
+#endif
+
 __device__ __forceinline__ float silu(float g) { return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)); }
 
 // Tile configuration.  BKB = bytes of K per row per tile (64 bf16 or 128 fp8 = 128 B,
@@ -307,14 +331,18 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
                 for (int r = 0; r < 4; ++r)
                   if (f + r < a.N) orow[f + r] = v[r];
             } else {
-              out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(sid) * a.ldo;
               out4 o;
 #pragma unroll
               for (int r = 0; r < 4; ++r) o[r] = static_cast<out_t>(v[r]);
-              if (f + 3 < a.N) *reinterpret_cast<out4*>(orow + f) = o;
-              else
-                for (int r = 0; r < 4; ++r)
-                  if (f + r < a.N) orow[f + r] = o[r];
+              if (a.add_div) {  // top-k combine in the epilogue (the launcher requires N % 4 == 0)
+                if (f < a.N) atomic_add4(static_cast<out_t*>(a.out) + static_cast<int64_t>(sid / a.add_div) * a.ldo + f, o);
+              } else {
+                out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(sid) * a.ldo;
+                if (f + 3 < a.N) *reinterpret_cast<out4*>(orow + f) = o;
+                else
+                  for (int r = 0; r < 4; ++r)
+                    if (f + r < a.N) orow[f + r] = o[r];
+              }
             }
           }
       }

@@ -160,7 +160,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
   // one fragment buffer for fp8 (8-register fragments) and for the 256-row tile on 16x16 MFMAs (twelve fragments
   // per K-step next to 128 accumulators), two otherwise
-  constexpr bool SINGLE = E::SCALED || (C::TILE == 16 && BT == 256);
+  constexpr bool SINGLE = E::SCALED || (C::TILE == 16 && BT >= 256);
   // fp8 epilogue: scales fetched up front where the registers allow it (the 256-row tile keeps 128 accumulators
   // and two address sets alive: measured 603 us with, 589 us without for the down projection at M = 4096; the
   // 128-row tile gains 2-5 %)
@@ -429,7 +429,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     if (!(ISS_)) {                                                                                         \
       bool any_ = false;                                                                                   \
       _Pragma("unroll") for (int r0_ = 0; r0_ < C::TT; r0_ += kWave)                                       \
-        any_ |= a.sorted[pid_t * BT + wt * C::TT + r0_ + lane] < a.num_valid;                              \
+        any_ |= r0_ + lane < C::TT && a.sorted[pid_t * BT + wt * C::TT + r0_ + lane] < a.num_valid;        \
       on_ = __ballot(any_) != 0;                                                                           \
       if (on_) FR_READ_FRAGS(sl, 0, 0)                                                                     \
     }                                                                                                      \
@@ -585,7 +585,8 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(const GemmArgs a, int n
         out4 o;
 #pragma unroll
         for (int r = 0; r < 4; ++r) o[r] = static_cast<out_t>(sum[r] * rw);
-        *reinterpret_cast<out4*>(static_cast<out_t*>(a.out) + at) = o;
+        if (a.add_div) atomic_add4(static_cast<out_t*>(a.out) + static_cast<int64_t>(sid / a.add_div) * a.ldo + pid_f * BF + cg * 4, o);
+        else *reinterpret_cast<out4*>(static_cast<out_t*>(a.out) + at) = o;
       }
     } else {
       f32x4 g = *reinterpret_cast<const f32x4*>(src), u = *reinterpret_cast<const f32x4*>(src + BF / 2);

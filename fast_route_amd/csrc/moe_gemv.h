@@ -379,6 +379,12 @@ __global__ void __launch_bounds__(kDownWaves * kWave) down_rows_kernel(GemmArgs 
                                                    static_cast<int64_t>(__builtin_amdgcn_readlane(t_slot, p)) * a.ldx + kofs + c * 512);
     }
   const int h_begin = blockIdx.x * hpw, h_end = min(h_begin + hpw, a.N);
+  if (ng == 0) {  // no valid pair at all (every id out of range): the sum over nothing is zero
+    for (int i = threadIdx.x; i < tokens * (h_end - h_begin); i += blockDim.x)
+      static_cast<typename Elem<T>::out_t*>(a.out)[static_cast<int64_t>(i / (h_end - h_begin)) * a.ldo + h_begin + i % (h_end - h_begin)] =
+          static_cast<typename Elem<T>::out_t>(0.f);
+    return;
+  }
   const int rounds = (h_end - h_begin + HB - 1) / HB, steps = rounds * ng;
   float acc[HB][NP];
 #pragma unroll

@@ -702,3 +702,67 @@ def test_random_shapes_against_oracle(native):
         out = fused_moe(x.cuda(), w1.cuda(), w2.cuda(), logits.cuda(), k, renorm)
         torch.cuda.synchronize()
         _assert_close(out, oracle.fused_moe(x, w1, w2, logits, k, renorm), dtype, f"random case {case}")
+
+
+@pytest.mark.parametrize("M,E,k,H,Fd", [(2, 8, 2, 512, 4096), (3, 8, 2, 512, 1024), (300, 8, 2, 512, 1024), (700, 8, 2, 512, 1024),
+                                        (200, 64, 6, 512, 384)])
+def test_out_of_range_expert_ids_are_dropped_pairs(native, M, E, k, H, Fd):
+    """Expert ids outside [0, E) (masked pairs of an expert-parallel caller) get no slot in the routing arrays
+    and contribute nothing: the oracle's per-expert masks never match them either (perf_test_moe.py:22-27).
+    Covers the decode kernels, the combine in the GEMM epilogue (top-2) and the combine kernel (top-6);
+    with every pair masked the output is exactly zero."""
+    from fast_route_amd import fused_experts
+    dtype = torch.bfloat16
+    _say(f"masked ids M={M} E={E} k={k}")
+    x, logits, w1, w2 = _inputs(M, H, Fd, E, 31, dtype)
+    tw, ti = oracle.gating_topk(logits, k, True)
+    g = torch.Generator().manual_seed(M)
+    drop = torch.rand(M, k, generator=g) < 0.3
+    ti = ti.clone()
+    ti[drop] = torch.where(torch.rand(int(drop.sum()), generator=g) < 0.5, -1, E + 3).int()
+    xd, w1d, w2d = x.cuda(), w1.cuda(), w2.cuda()
+    out = fused_experts(xd, w1d, w2d, tw.cuda(), ti.cuda())
+    torch.cuda.synchronize()
+    _assert_close(out, oracle.moe_experts(x, w1, w2, tw, ti), dtype, f"masked ids M={M}")
+    none = torch.full_like(ti, -1)
+    out0 = fused_experts(xd, w1d, w2d, tw.cuda(), none.cuda())
+    torch.cuda.synchronize()
+    assert torch.count_nonzero(out0) == 0, "all pairs masked: output must be zero"
+
+
+@pytest.mark.parametrize("E", [8, 100, 256])
+@pytest.mark.parametrize("M", [3, 40])
+def test_nan_logit_rows_do_not_reach_the_weights(native, E, M):
+    """A token whose router logits are all NaN has no valid expert (with more than 64 experts the gating core
+    leaves an id outside [0, E) behind): its pairs are dropped by the routing - also by the routing done inside
+    the decode gate/up launch - instead of indexing the weights, and the other tokens are unaffected."""
+    from fast_route_amd import fused_moe
+    dtype = torch.bfloat16
+    _say(f"NaN logits E={E} M={M}")
+    x, logits, w1, w2 = _inputs(M, 2048, 256, E, 13, dtype)
+    logits = logits.clone()
+    logits[1, :] = float("nan")
+    out = fused_moe(x.cuda(), w1.cuda(), w2.cuda(), logits.cuda(), 2, True)
+    torch.cuda.synchronize()
+    keep = [m for m in range(M) if m != 1]
+    ref = oracle.fused_moe(x[keep], w1, w2, logits[keep], 2, True)
+    _assert_close(out[keep], ref, dtype, f"NaN logits E={E}")
+    if E > 64:
+        assert torch.count_nonzero(out[1]) == 0
+
+
+@pytest.mark.parametrize("M", [40, 300, 3000])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_top2_combine_in_the_epilogue_is_deterministic(native, M, dtype):
+    """Top-2 layers add the two weighted rows of a token into a zero-filled output with packed atomics; the
+    result may not depend on which pair arrives first: same bits on every run, also in place."""
+    from fast_route_amd import fused_moe
+    _say(f"top-2 epilogue combine M={M} {dtype}")
+    x, logits, w1, w2 = _inputs(M, 512, 1024, 8, 17, dtype)
+    xd, w1d, w2d, ld = x.cuda(), w1.cuda(), w2.cuda(), logits.cuda()
+    first = fused_moe(xd, w1d, w2d, ld, 2, True)
+    for _ in range(4):
+        assert torch.equal(fused_moe(xd, w1d, w2d, ld, 2, True), first)
+    xin = xd.clone()
+    assert torch.equal(fused_moe(xin, w1d, w2d, ld, 2, True, inplace=True), first)
+    _assert_close(first, oracle.fused_moe(x, w1, w2, logits, 2, True), dtype, f"top-2 M={M}")
