@@ -538,6 +538,7 @@ def main():
                                % (args.shape, H, F, E, topk, args.tokens, args.dtype),
                    "tokens": args.tokens, "hidden": H, "ffn": F, "experts": E, "topk": topk, "seed": args.seed,
                    "flops_formula": "6*M*topk*H*F"},
+        "native_library": os.path.basename(N.LIB_PATH),
         "layer_roofline_frac": head["roofline_frac"], "layer_bound": head["bound"],
         "stage_us": head["stage_us"],
         "roofline": kernel_roofline(shape, head, fp8 is not None),

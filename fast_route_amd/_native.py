@@ -6,7 +6,8 @@ import os
 from ctypes import c_char_p, c_int, c_int32, c_int64, c_void_p
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libfast_route_hip.so")
+# FR_NATIVE_LIB: another build of the library (a measurement build, see build.py); bench.py records which one ran
+LIB_PATH = os.environ.get("FR_NATIVE_LIB") or os.path.join(HERE, "libfast_route_hip.so")
 
 FR_F16, FR_BF16, FR_F32, FR_FP8_E4M3, FR_I32, FR_I64 = range(6)
 FR_W1_TILED, FR_W2_TILED, FR_W_TILED = 0x100, 0x200, 0x300  # OR-ed into a dtype argument: w1 / w2 / both are in the layout of fr_moe_prepare_weights
@@ -20,7 +21,8 @@ class FrMoePlan(ctypes.Structure):
 
 
 class FrMoeTunables(ctypes.Structure):
-    _fields_ = [("block", c_int32), ("split_k", c_int32), ("group_m", c_int32), ("no_tail_split", c_int32)]
+    _fields_ = [("block", c_int32), ("split_k", c_int32), ("group_m", c_int32), ("no_tail_split", c_int32),
+                ("epilogue_combine", c_int32)]
 
 
 # name -> (restype, argtypes); must list every symbol the header declares

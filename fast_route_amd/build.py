@@ -39,13 +39,20 @@ def _run(cmd):
     return out
 
 
+MEASUREMENT_LIB = os.path.join(HERE, "libfast_route_hip_measure.so")
+
+
 def build(verbose: bool = False) -> str:
     """Compiles every source and links the shared library; returns its path.
     FR_HIPCC_FLAGS in the environment adds compiler flags (the measurement switches of
-    csrc/moe_gemm_persistent.h, e.g. FR_HIPCC_FLAGS="-DFR_ABL_NOLOAD")."""
+    csrc/moe_gemm_persistent.h, e.g. FR_HIPCC_FLAGS="-DFR_ABL_NOLOAD": kernels whose RESULTS ARE WRONG,
+    only their timings mean something).  Such a build never replaces the library tests and callers load:
+    it goes to libfast_route_hip_measure.so (objects under build_measure/), which _native loads only when
+    FR_NATIVE_LIB names it."""
     hipcc = _hipcc()
     extra = os.environ.get("FR_HIPCC_FLAGS", "").split()
-    objdir = os.path.join(HERE, "build")
+    objdir = os.path.join(HERE, "build_measure" if extra else "build")
+    lib = MEASUREMENT_LIB if extra else LIB
     os.makedirs(objdir, exist_ok=True)
     objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
 
@@ -57,8 +64,8 @@ def build(verbose: bool = False) -> str:
         for out in pool.map(one, zip(SOURCES, objs)):
             if verbose and out.strip():
                 print(out)
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
-    return LIB
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *objs])
+    return lib
 
 
 if __name__ == "__main__":

@@ -38,6 +38,9 @@ int gateup_rows_routed(const void* x, const void* w1, const void* logits, int lo
                        int64_t F, int E, int topk, int renorm, int block, int dtype, void* act, float* topk_w,
                        int32_t* topk_ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost, hipStream_t st);
 
+// Looks up (once per device) the device address of the static scratch behind fr_fused_moe_noalloc on the current device.
+int prepare_static_scratch();
+
 // Down projection + routed weight + top-k combine (what fr_moe_down_combine / fr_moe_down_combine_fp8 launch).  pair_ids:
 // the [M, topk] expert ids, or nullptr; with them a pair whose id lies outside [0, E) - it has no slot in the routing
 // arrays - contributes nothing to its token's sum (without them its never-written partial row would be added).

@@ -56,7 +56,7 @@ Carve carve(void* base, int64_t M, int64_t H, int64_t F, int E, int topk, int dt
   return c;
 }
 
-fr_moe_tunables g_tunables = {0, 0, 0, 0};
+fr_moe_tunables g_tunables = {0, 0, 0, 0, 0};
 
 int check_layer_shapes(const char* who, int64_t M, int64_t H, int64_t F, int E, int topk, int dtype) {
   FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16 || dtype == FR_FP8_E4M3, FR_E_DTYPE, "%s: dtype %d not in {f16, bf16, fp8_e4m3}", who, dtype);
@@ -76,7 +76,7 @@ using namespace fr;
 
 extern "C" int fr_moe_set_tunables(const fr_moe_tunables* t) {
   if (!t) {
-    g_tunables = fr_moe_tunables{0, 0, 0, 0};
+    g_tunables = fr_moe_tunables{0, 0, 0, 0, 0};
     return FR_OK;
   }
   FR_REQUIRE(t->block == 0 || t->block == 16 || t->block == 32 || t->block == 64 || t->block == 128 || t->block == 256,
@@ -84,6 +84,7 @@ extern "C" int fr_moe_set_tunables(const fr_moe_tunables* t) {
   FR_REQUIRE(t->split_k >= 0 && t->split_k <= 64, FR_E_SHAPE, "fr_moe_set_tunables: split_k=%d outside [0, 64]", t->split_k);
   FR_REQUIRE(t->group_m >= 0 && t->group_m <= 64, FR_E_SHAPE, "fr_moe_set_tunables: group_m=%d outside [0, 64]", t->group_m);
   FR_REQUIRE(t->no_tail_split == 0 || t->no_tail_split == 1, FR_E_SHAPE, "fr_moe_set_tunables: no_tail_split=%d", t->no_tail_split);
+  FR_REQUIRE(t->epilogue_combine == 0 || t->epilogue_combine == 1, FR_E_SHAPE, "fr_moe_set_tunables: epilogue_combine=%d", t->epilogue_combine);
   g_tunables = *t;
   return FR_OK;
 }
@@ -292,6 +293,10 @@ int static_scratch(void** out) {
   return FR_OK;
 }
 }  // namespace
+int prepare_static_scratch() {
+  void* p = nullptr;
+  return static_scratch(&p);
+}
 }  // namespace fr
 
 extern "C" int fr_fused_moe_noalloc(const void* x, const void* w1, const void* w2, const void* logits, int logits_dtype,

@@ -215,8 +215,8 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
   }
   if (splits == 1) {
     const int row_dtype = dtype == FR_F16 ? FR_F16 : FR_BF16;  // type a single slice's rows are written in
-    if (topk == 2 && out_dtype == row_dtype) {
-      // Two pairs per token: the combine happens in the GEMM epilogue.  `out` is zero-filled (by a kernel: the call
+    if (tunables().epilogue_combine && topk == 2 && out_dtype == row_dtype) {
+      // Two pairs per token, on request (measured slower than the combine kernel): the combine happens in the GEMM epilogue.  `out` is zero-filled (by a kernel: the call
       // stays capturable) and every pair's weighted row is added into its token's row with packed atomics - 0 + a
       // is exact and a + b is rounded once, so the result does not depend on which pair arrives first and equals
       // the sum the combine kernel would form from the same two rounded rows.  No partial rows, no combine launch;
@@ -369,6 +369,7 @@ extern "C" int fr_moe_prepare(int dtype) {
   } else {
     return fail(FR_E_DTYPE, "fr_moe_prepare: dtype %d not in {f16, bf16, fp8_e4m3}", dtype);
   }
+  if (rc == FR_OK) rc = prepare_static_scratch();  // fr_fused_moe_noalloc then has no set-up left either
   return rc;
 }
 

@@ -8,7 +8,11 @@
  *   - all pointers except `stream` are DEVICE addresses owned by the caller;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
  *   - every call only enqueues work on `stream`: no allocation, no host
- *     synchronisation, no device-to-host copy, safe under graph capture;
+ *     synchronisation, no device-to-host copy.  Under graph capture that holds once the
+ *     kernels are set up on the device: the first call of a tile configuration raises its
+ *     dynamic-LDS limit and queries its occupancy (set-up calls, not stream work), so a
+ *     caller whose first call would be captured calls fr_moe_prepare once per device and
+ *     dtype beforehand, or makes one eager call of the same shape;
  *   - return value 0 on success, a negative FR_E_* code otherwise;
  *     fr_last_error_string() gives the thread-local message of the last failure;
  *   - tensors are dense row-major unless a stride argument says otherwise.
@@ -141,7 +145,7 @@ int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk, int dtype,
 
 /* Per-device set-up of every grouped-GEMM kernel of `dtype` (FR_F16, FR_BF16, FR_FP8_E4M3) on the
  * CURRENT device: raises the kernels' dynamic-LDS limits and caches the persistent kernels'
- * occupancy.  The first call of each tile configuration does the same work lazily; a caller whose
+ * occupancy, and looks up the address of fr_fused_moe_noalloc's scratch.  The first call of each tile configuration does the same work lazily; a caller whose
  * first call would be under graph capture (set-up calls are not stream work) calls this once per
  * device and dtype beforehand.  Launches nothing.  No counterpart in the reference (Triton compiles
  * and configures its kernels on first use, fast_route/fast_route/layers/stable_route.py:67). */
@@ -156,6 +160,12 @@ int fr_moe_prepare(int dtype);
  *   group_m    token blocks walked together over the feature tiles (L2 sharing of weight tiles),
  *              1..64
  *   no_tail_split  1: never split the last, partly filled round of tiles along K
+ *   epilogue_combine  1: with two experts per token and one K slice, the down GEMM adds each pair's
+ *              weighted row into a zero-filled `out` with packed atomic adds in its epilogue (the sum of
+ *              two rows does not depend on their order) instead of writing the pairs' rows for the
+ *              combine kernel.  Off by default: measured slower - 16.7 M four-byte atomics at Mixtral
+ *              shape and 4096 tokens cost the down stage 1015 us against 900 us (3650 against 3200 us at
+ *              16384 tokens, 149 against 146 us at 16 tokens)
  * fr_moe_get_plan, fr_fused_moe, fr_fused_experts, fr_fused_moe_fp8 and the staged GEMM entry
  * points all see them.  fr_moe_set_tunables(NULL) restores the defaults.
  * Replaces: the per-GEMM config dictionaries edited by hand in the reference's tile study
@@ -166,6 +176,7 @@ typedef struct fr_moe_tunables {
   int32_t split_k;
   int32_t group_m;
   int32_t no_tail_split;
+  int32_t epilogue_combine;
 } fr_moe_tunables;
 int fr_moe_set_tunables(const fr_moe_tunables* t);
 int fr_moe_get_tunables(fr_moe_tunables* t);
@@ -224,8 +235,9 @@ int fr_fused_moe(const void* x, const void* w1, const void* w2, const void* logi
  * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc.  Sizes whose fr_moe_get_plan().workspace_bytes exceed 64 MiB are
  * rejected with FR_E_WORKSPACE (Mixtral-8x7B shape: up to 207 tokens).  The array's
- * device address is looked up on the first call on each device (with that device
- * current); nothing in the array has to start at zero.  All calls on one GPU share the
+ * device address is looked up by fr_moe_prepare, or else on the first call on each device
+ * (with that device current): before capturing a call, call fr_moe_prepare or make one
+ * eager call on that device.  Nothing in the array has to start at zero.  All calls on one GPU share the
  * array: calls that overlap in time on one GPU (two streams, two threads) race. */
 int fr_fused_moe_noalloc(const void* x, const void* w1, const void* w2, const void* logits,
                          int logits_dtype, int64_t M, int64_t H, int64_t F, int E, int topk,

@@ -154,7 +154,7 @@ def test_tunables_override_the_plan_and_reset():
         fr.set_tunables(block=128, split_k=3)
         p = plan(4096)
         assert (p.block, p.split_k) == (128, 3) and p.sorted_len == 8192 + 8 * 127
-        assert fr.get_tunables() == {"block": 128, "split_k": 3, "group_m": 0, "no_tail_split": False}
+        assert fr.get_tunables() == {"block": 128, "split_k": 3, "group_m": 0, "no_tail_split": False, "epilogue_combine": False}
         with fr.tunables(no_tail_split=True):
             assert plan(4096).tail_bytes == 0 and plan(4096).block == 256  # the context replaces, then restores
         assert plan(4096).block == 128

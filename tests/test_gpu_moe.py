@@ -754,15 +754,90 @@ def test_nan_logit_rows_do_not_reach_the_weights(native, E, M):
 @pytest.mark.parametrize("M", [40, 300, 3000])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_top2_combine_in_the_epilogue_is_deterministic(native, M, dtype):
-    """Top-2 layers add the two weighted rows of a token into a zero-filled output with packed atomics; the
-    result may not depend on which pair arrives first: same bits on every run, also in place."""
+    """The epilogue_combine knob: top-2 layers add the two weighted rows of a token into a zero-filled output
+    with packed atomics.  The result may not depend on which pair arrives first: same bits on every run, also
+    in place, and the same bits as the combine kernel forms from the same two rounded rows."""
+    import fast_route_amd as fr
     from fast_route_amd import fused_moe
     _say(f"top-2 epilogue combine M={M} {dtype}")
     x, logits, w1, w2 = _inputs(M, 512, 1024, 8, 17, dtype)
     xd, w1d, w2d, ld = x.cuda(), w1.cuda(), w2.cuda(), logits.cuda()
-    first = fused_moe(xd, w1d, w2d, ld, 2, True)
-    for _ in range(4):
-        assert torch.equal(fused_moe(xd, w1d, w2d, ld, 2, True), first)
-    xin = xd.clone()
-    assert torch.equal(fused_moe(xin, w1d, w2d, ld, 2, True, inplace=True), first)
+    with fr.tunables(split_k=1):
+        by_kernel = fused_moe(xd, w1d, w2d, ld, 2, True)
+    with fr.tunables(split_k=1, epilogue_combine=True):
+        first = fused_moe(xd, w1d, w2d, ld, 2, True)
+        for _ in range(4):
+            assert torch.equal(fused_moe(xd, w1d, w2d, ld, 2, True), first)
+        xin = xd.clone()
+        assert torch.equal(fused_moe(xin, w1d, w2d, ld, 2, True, inplace=True), first)
+    torch.cuda.synchronize()
     _assert_close(first, oracle.fused_moe(x, w1, w2, logits, 2, True), dtype, f"top-2 M={M}")
+    assert torch.equal(first, by_kernel), "epilogue combine and combine kernel round differently"
+
+
+_FIRST_CALL_CAPTURE = r'''
+import sys
+sys.path.insert(0, sys.argv[1])
+import torch
+import fast_route_amd as fr
+from fast_route_amd import _native as N
+from fast_route_amd.layers.fused_moe import plan
+
+dtype, lib = torch.bfloat16, N.lib()
+fr.prepare(dtype)                      # every kernel set up, the no-alloc scratch resolved: nothing left to do lazily
+gen = torch.Generator().manual_seed(9)
+cases = []
+for M, H, Fd, E, k in ((2, 4096, 512, 4, 2), (16, 1024, 2048, 4, 2), (1536, 1024, 2048, 4, 2)):
+    x = torch.randn(M, H, generator=gen).to(dtype).cuda()
+    logits = torch.randn(M, E, generator=gen).cuda()
+    w1 = (torch.randn(E, 2 * Fd, H, generator=gen) * 0.02).to(dtype).cuda()
+    w2 = (torch.randn(E, H, Fd, generator=gen) * 0.02).to(dtype).cuda()
+    p = plan(M, H, Fd, E, k, dtype)
+    ws = torch.empty(max(p.workspace_bytes, 256), dtype=torch.uint8, device="cuda")
+    out, out_na = torch.zeros(M, H, dtype=dtype, device="cuda"), torch.zeros(M, H, dtype=dtype, device="cuda")
+    na = p.workspace_bytes <= (64 << 20)
+
+    def call(stream, x=x, w1=w1, w2=w2, logits=logits, M=M, H=H, Fd=Fd, E=E, k=k, out=out, out_na=out_na, ws=ws, na=na):
+        N.check(lib.fr_fused_moe(x.data_ptr(), w1.data_ptr(), w2.data_ptr(), logits.data_ptr(), N.FR_F32, M, H, Fd, E, k, 1,
+                                 N.FR_BF16, out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+        if na:
+            N.check(lib.fr_fused_moe_noalloc(x.data_ptr(), w1.data_ptr(), w2.data_ptr(), logits.data_ptr(), N.FR_F32, M, H, Fd,
+                                             E, k, 1, N.FR_BF16, out_na.data_ptr(), stream))
+    cases.append((M, call, out, out_na, na))
+torch.cuda.synchronize()
+graphs = []
+for M, call, out, out_na, na in cases:  # the captured calls are this process's first launches of these kernels
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        call(torch.cuda.current_stream().cuda_stream)
+    graphs.append(g)
+for (M, call, out, out_na, na), g in zip(cases, graphs):
+    for rep in range(2):
+        out.zero_(); out_na.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got, got_na = out.clone(), out_na.clone()
+        out.zero_(); out_na.zero_()
+        call(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert torch.count_nonzero(got) > 0
+        assert torch.equal(got, out), "M=%d replay %d: captured first call differs from the eager call" % (M, rep)
+        if na:
+            assert torch.equal(got_na, out_na) and torch.equal(got_na, got), "M=%d: no-alloc entry under capture" % M
+print("FIRST-CALL-CAPTURE-OK")
+'''
+
+
+def test_first_call_under_graph_capture_after_prepare(native):
+    """What fr_moe_prepare exists for: in a fresh process, after fr_moe_prepare and nothing else, the whole layer -
+    through fr_fused_moe and through fr_fused_moe_noalloc - is captured as the process's FIRST launch of its
+    kernels (weight-row decode kernels, decode tiles with the fused route+align launch, persistent tiles with
+    their last-round split) and replays to the bits of the eager calls made afterwards."""
+    import os
+    import subprocess
+    _say("first call captured after fr_moe_prepare (fresh process)")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, "-c", _FIRST_CALL_CAPTURE, root], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                          text=True, timeout=110)
+    assert proc.returncode == 0 and "FIRST-CALL-CAPTURE-OK" in proc.stdout, proc.stdout[-3000:]
