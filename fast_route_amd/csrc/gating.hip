@@ -65,7 +65,7 @@ __global__ __launch_bounds__(kGateThreads) void gating_topk_blocked_kernel(
 // expert-major LDS rows (two K rows packed per 32-bit store) that the MFMA "A" operand reads
 // as 16-byte vectors; token rows come straight from HBM as the "B" operand, fetched for the
 // whole chunk before the barrier that publishes it.
-constexpr int kRgMaxE = 64;
+constexpr int kRgMaxE = 128;  // the reference's own bound (ops/stable_route.py:134)
 
 template <typename T> struct Mfma16;
 template <> struct Mfma16<bf16_t> {
@@ -79,22 +79,28 @@ template <> struct Mfma16<f16_t> {
 
 // KC = K rows of the gate per LDS chunk; TT = 16-token tiles per wavefront in the unsplit form (many
 // experts: more tokens per transposed gate chunk).
-template <typename T, int G, bool SPLITK, int KC, int TT>
+// G lanes gate a token, VPL logits each: up to G * VPL experts (VPL = 2: 65..128 experts).
+template <typename T, int G, bool SPLITK, int KC, int TT, int VPL = 1>
 __global__ __launch_bounds__(kGateThreads) void route_gate_kernel(
     const T* __restrict__ hidden, const T* __restrict__ gate, int64_t M, int H, int E, int topk,
     int renorm, float* __restrict__ w_out, int32_t* __restrict__ ids_out) {
   typedef typename Mfma16<T>::vec8 vec8;
   static_assert(kGateThreads == 256, "4 wavefronts");
   static_assert(!SPLITK || TT == 1, "the split form has one token tile");
-  constexpr int ET = (G + 15) / 16;              // expert tiles of 16
+  constexpr int ET = (G * VPL + 15) / 16;        // expert tiles of 16
   constexpr int TPC = SPLITK ? 16 : 64 * TT;     // tokens per workgroup
   constexpr int KW = SPLITK ? KC / 4 : KC;       // K elements of a chunk one wavefront multiplies
   constexpr int KSTEPS = KW / 32;
   constexpr int PITCH = KC + 8;                  // elements; keeps 16-byte alignment, spreads banks
   constexpr int LP = ET * 16 + 1;                // pitch of a logit row (floats)
-  __shared__ __attribute__((aligned(16))) T gt[ET * 16 * PITCH];
-  __shared__ float logit[TPC * LP];
-  __shared__ float part[SPLITK ? 4 * 16 * LP : 1];
+  // the transposed gate chunk during the K loop; afterwards the same memory holds the logits (and the K slices' partial sums)
+  constexpr int GT_BYTES = ET * 16 * PITCH * static_cast<int>(sizeof(T));
+  constexpr int LG_BYTES = (TPC * LP + (SPLITK ? 4 * 16 * LP : 0)) * 4;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[GT_BYTES > LG_BYTES ? GT_BYTES : LG_BYTES];
+  static_assert(sizeof(smem) <= 65536, "LDS");
+  T* gt = reinterpret_cast<T*>(smem);
+  float* logit = reinterpret_cast<float*>(smem);
+  float* part = logit + TPC * LP;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * TPC;
   const int kw0 = SPLITK ? wave * KW : 0;        // the wavefront's K range inside a chunk
@@ -162,6 +168,7 @@ __global__ __launch_bounds__(kGateThreads) void route_gate_kernel(
         for (int t = 0; t < TT; ++t) acc[t][j] = Mfma16<T>::mma(gf, xf[t][ks], acc[t][j]);
       }
   }
+  __syncthreads();  // every wavefront has read its last gate chunk: the memory becomes the logit rows
   // accumulator rows are experts (lane/16*4 + r inside tile j), columns tokens
   float* dst = SPLITK ? part + wave * 16 * LP : logit;
 #pragma unroll
@@ -183,8 +190,8 @@ __global__ __launch_bounds__(kGateThreads) void route_gate_kernel(
     const int64_t token = tok0 + t;
     const bool live = token < M;
     const float* row = logit + t * LP;
-    gate_token<G, 1>([&](int e) { return row[e]; }, live, E, topk, renorm, w_out + token * topk,
-                     ids_out + token * topk);
+    gate_token<G, VPL>([&](int e) { return row[e]; }, live, E, topk, renorm, w_out + token * topk,
+                       ids_out + token * topk);
   }
 }
 
@@ -260,19 +267,20 @@ extern "C" int fr_gating_topk(const void* logits, int logits_dtype, int64_t M, i
 
 namespace fr {
 namespace {
-template <typename T, int G>
+template <typename T, int G, int VPL = 1>
 void launch_route_gate(const void* hidden, const void* gate, int64_t M, int H, int E, int topk, int renorm,
                        float* w, int32_t* ids, hipStream_t st) {
-  constexpr int ET = (G + 15) / 16;
+  constexpr int ET = (G * VPL + 15) / 16;
   // 64 (128 with many experts) tokens per workgroup once that gives every CU a workgroup or two; below,
   // 16 tokens with K split over the wavefronts (more workgroups, a quarter of the row per wavefront)
   if (M >= 16384) {
-    constexpr int TT = ET >= 2 ? 2 : 1;
-    hipLaunchKernelGGL((route_gate_kernel<T, G, false, 256, TT>), dim3(static_cast<unsigned>(ceil_div(M, 64 * TT))), dim3(kGateThreads),
+    constexpr int TT = (ET >= 2 && VPL == 1) ? 2 : 1;
+    constexpr int KCU = VPL == 1 ? 256 : 128;  // 128 expert rows of 256 K elements would not fit the LDS
+    hipLaunchKernelGGL((route_gate_kernel<T, G, false, KCU, TT, VPL>), dim3(static_cast<unsigned>(ceil_div(M, 64 * TT))), dim3(kGateThreads),
                        0, st, static_cast<const T*>(hidden), static_cast<const T*>(gate), M, H, E, topk, renorm, w, ids);
   } else {
-    constexpr int KC = 256;  // longer chunks for few experts leave fewer workgroups per CU: slower at M = 8192, no gain at M = 1
-    hipLaunchKernelGGL((route_gate_kernel<T, G, true, KC, 1>), dim3(static_cast<unsigned>(ceil_div(M, 16))), dim3(kGateThreads), 0, st,
+    constexpr int KC = VPL == 1 ? 256 : 128;  // longer chunks for few experts leave fewer workgroups per CU: slower at M = 8192, no gain at M = 1
+    hipLaunchKernelGGL((route_gate_kernel<T, G, true, KC, 1, VPL>), dim3(static_cast<unsigned>(ceil_div(M, 16))), dim3(kGateThreads), 0, st,
                        static_cast<const T*>(hidden), static_cast<const T*>(gate), M, H, E, topk, renorm, w, ids);
   }
 }
@@ -285,7 +293,8 @@ int dispatch_route_gate(const void* hidden, const void* gate, int64_t M, int H, 
   else if (E <= 8) launch_route_gate<T, 8>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
   else if (E <= 16) launch_route_gate<T, 16>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
   else if (E <= 32) launch_route_gate<T, 32>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
-  else launch_route_gate<T, 64>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
+  else if (E <= 64) launch_route_gate<T, 64>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
+  else launch_route_gate<T, 64, 2>(hidden, gate, M, H, E, topk, renorm, w, ids, st);
   return check_launch("route_gate_kernel");
 }
 }  // namespace

@@ -52,7 +52,7 @@ def fused_route(hidden_state: torch.Tensor, gate: torch.Tensor, topk: int, topk_
     M, K = hidden_state.shape
     K2, E = gate.shape
     assert K == K2, "Incompatible dimensions"
-    assert E <= 256, f"{E} number of experts should be at most 256"
+    assert E <= 128, f"{E} number of experts should be small enough to reside in shared memory"  # ops/stable_route.py:134
     assert hidden_state.dtype in (torch.float16, torch.bfloat16) and gate.dtype == hidden_state.dtype
     w_view, i_view = _out_views(topk_weights, topk_ids, M, topk)
     dev = hidden_state.device
@@ -60,13 +60,13 @@ def fused_route(hidden_state: torch.Tensor, gate: torch.Tensor, topk: int, topk_
     # fp16 weights and int64 ids, tests/test_route.py:30-38) are filled by a cast of dense temporaries
     w_k = w_view if w_view.dtype == torch.float32 else torch.empty((M, topk), dtype=torch.float32, device=dev)
     i_k = i_view if i_view.dtype == torch.int32 else torch.empty((M, topk), dtype=torch.int32, device=dev)
-    if E <= 64 and K % 8 == 0 and hidden_state.is_contiguous() and gate.is_contiguous():
+    if K % 8 == 0 and hidden_state.is_contiguous() and gate.is_contiguous():
         N.check(N.lib().fr_route_gate(hidden_state.data_ptr(), gate.data_ptr(), N.dtype_code(hidden_state.dtype),
                                       M, K, E, topk, int(bool(renormalize)), w_k.data_ptr(), i_k.data_ptr(),
                                       N.stream_ptr(dev)))
     else:
-        # more than 64 experts (or strided operands): logits accumulated AND kept in fp32, as the reference's
-        # kernel keeps its accumulator (ops/stable_route.py:66-97), then the same stable top-k
+        # strided operands or K % 8 != 0 (shapes the reference's asserts refuse anyway): logits accumulated AND kept in
+        # fp32, as the reference's kernel keeps its accumulator (ops/stable_route.py:66-97), then the same stable top-k
         logits = torch.matmul(hidden_state.float(), gate.float())
         _gating(logits, topk, renormalize, w_k, i_k)
     if w_k is not w_view:

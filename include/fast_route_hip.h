@@ -65,7 +65,8 @@ int fr_gating_topk(const void* logits, int logits_dtype, int64_t M, int64_t E, i
 /* Gate-matrix form: logits = hidden[M, H] @ gate[H, E] accumulated in fp32,
  * then fr_gating_topk, in one kernel (no [M, E] round trip).
  * Replaces: fused_route, fast_route/fast_route/ops/stable_route.py:123-178.
- * Limits: E <= 64, H % 8 == 0; dtype in {FR_F16, FR_BF16}. */
+ * Limits: E <= 128 (the reference's bound, ops/stable_route.py:134), H % 8 == 0;
+ * dtype in {FR_F16, FR_BF16}. */
 int fr_route_gate(const void* hidden, const void* gate, int dtype, int64_t M, int64_t H, int64_t E,
                   int topk, int renormalize, float* weights_out, int32_t* ids_out, void* stream);
 

@@ -129,7 +129,7 @@ def test_route_gate_fused_gemm(native, E, topk, H, dtype):
         torch.testing.assert_close(w.cpu()[ok], ow[ok], atol=1e-4, rtol=0)
 
 
-@pytest.mark.parametrize("E,topk,H", [(8, 2, 264), (64, 6, 256), (24, 3, 512)])
+@pytest.mark.parametrize("E,topk,H", [(8, 2, 264), (64, 6, 256), (24, 3, 512), (128, 8, 256), (100, 6, 512)])
 def test_route_gate_large_batch(native, E, topk, H):
     """From 16384 tokens on the kernel takes its unsplit form (64 or 128 tokens per workgroup,
     every wavefront the whole K range of its own tokens); 16500 tokens leave a ragged last
