@@ -20,7 +20,13 @@ namespace {
 constexpr int kSmallThreads = 1024;
 constexpr int kSmallWaves = kSmallThreads / kWave;
 constexpr int kSmallMaxE = 256;
-constexpr int64_t kSmallMaxN = 8192;  // above, the three-launch path is faster (measured 9.4 vs ~10 us here, 15.7 vs 9.8 us at 16384)
+// One workgroup sorts up to this many pairs; above, two launches spread over the CUs are faster.  Measured, gating +
+// sort back to back, one workgroup against two launches: 4096 pairs 12.9 / 14.7 us (8 experts), 15.2 / 16.1 (64 experts);
+// 8192 pairs 16.2 / 15.4 and 20.0 / 17.7 us.
+constexpr int64_t kSmallMaxN = 6144;
+// Gating and sort in ONE launch up to this many pairs (above, the gating kernel spread over the CUs plus the
+// one-workgroup sort win: 2048 pairs 31.6 against 29.5 us for a small layer, 1536 pairs on 64 experts 51.8 against 26.5)
+constexpr int64_t kRouteAlignMaxN = 1024;
 constexpr int kMaxE = 1024;
 constexpr int kSegThreads = 256;
 constexpr int kSegWaves = kSegThreads / kWave;
@@ -484,7 +490,7 @@ void dispatch_route_align(const void* logits, int64_t M, int E, int topk, int re
 // (one workgroup gates and sorts 1024 pairs in 10.5 us; from there on the gating kernel spread over the CUs
 // plus the one-workgroup sort are faster: 8.9 us + a launch gap at 1024 pairs, 12.6 against 26.8 us at 4096)
 bool route_align_fits(int64_t M, int E, int topk) {
-  return M >= 1 && M * topk <= 1024 && use_small_path(M * topk, E) && M * E <= 16384 && topk <= E;
+  return M >= 1 && M * topk <= kRouteAlignMaxN && use_small_path(M * topk, E) && M * E <= 16384 && topk <= E;
 }
 int route_align_small(const void* logits, int logits_dtype, int64_t M, int E, int topk, int renorm, int block,
                       float* w, int32_t* ids, int32_t* sorted, int32_t* expert_ids, int32_t* npost,

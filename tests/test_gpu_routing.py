@@ -77,7 +77,7 @@ def test_align_routing_stress_config(native, B):
 
 
 def test_align_medium_sizes_cross_path_boundary(native):
-    for n_tokens in (2730, 2731, 8192, 20000):
+    for n_tokens in (1024, 1025, 1365, 1366, 2730, 2731, 8192, 20000):  # 6144 / 6150 pairs straddle the one-workgroup limit
         _say(f"align boundary M={n_tokens}")
         rng = np.random.default_rng(n_tokens)
         ids = rng.integers(0, 64, size=(n_tokens, 6)).astype(np.int32)
