@@ -454,22 +454,114 @@ def other_configs(torch, N, args, mixtral_weights):
                   "peak_tflops": PEAK_FP8_TFLOPS, "sweep": sweep,
                   "vs_oracle_M4096": oracle_error(torch, shape, layer, 24, fp8=fp8)}
     del fp8, layer
+    # Mixtral shape again with the down-projection weights in the prepared layout (prepare_weights, its default)
+    from fast_route_amd import prepare_weights
+    _, w2p, flags = prepare_weights(w1, w2, "w2")
+    sweep = []
+    for M in (16, 256, 1024, 4096, 16384):
+        rec, layer = measure(torch, N, shape, M, w1, w2p, steps, warmup, args.seed, prepared=flags)
+        sweep.append(dict(compact(rec), stage_us=rec["stage_us"]))
+    out["prepared_w2"] = {"workload": "Mixtral shape bf16, w2 re-laid-out once by prepare_weights (64-row x 128-byte tiles); w1 as the reference has it",
+                          "sweep": sweep, "vs_oracle_M16384": oracle_error(torch, shape, layer)}
+    del w2p, layer
     return out
 
 
 def reference_protocol(torch, N, args):
     """The reference's own benchmark protocol (benchmarks/fused_route/moe_bench.py:10-38,53,83-99): fp16 operands
-    drawn as randn / 10, shape from -n (ffn) -k (hidden) -e --topk, m = 2^0 .. 2^14, and its "TFLOPS" figure
-    2*m*n*k / t (a sixth of the layer's real work at top-2) next to the real one."""
+    drawn as randn / 10, shape from -n (ffn) -k (hidden) -e --topk, m = 2^0 .. 2^14, the GATE-MATRIX layer
+    fused_moe(a, gate, w1, w2, topk, True, False) as the timed call (:92-94; routing GEMM, Python and allocations
+    included, as the reference times them), median of the repetitions (its do_bench quantile 0.5), and its "TFLOPS"
+    figure 2*m*n*k / t (a sixth of the layer's real work at top-2) next to the real one."""
+    from fast_route_amd.layers.stable_route import fused_moe as gate_matrix_layer
+    from fast_route_amd.layers.fused_moe import plan
     shape = dict(H=args.k, F=args.n, E=args.e, topk=args.topk, zipf=False)
     w1, w2 = make_weights(torch, shape, args.seed, torch.float16, 0.1)
+    g = torch.Generator(device="cuda").manual_seed(args.seed)
+    gate = (torch.randn(args.k, args.e, generator=g, device="cuda") / 10).half()
     rows = []
     for m in ([args.tokens] if args.no_sweep else [2 ** i for i in range(15)]):
-        rec, _ = measure(torch, N, shape, m, w1, w2, args.steps, args.warmup, args.seed, dtype=torch.float16, x_scale=0.1)
-        rows.append({"m": m, "us_per_layer": rec["us_per_layer"], "ref_2mnk_tflops": rec["ref_2mnk_tflops"],
-                     "tflops": rec["tflops"], "block": rec["block"]})
-    return {"protocol": "fp16, randn/10, n=%d k=%d e=%d topk=%d, mean of %d back-to-back steps" % (args.n, args.k, args.e, args.topk, args.steps),
+        a = (torch.randn(m, args.k, generator=g, device="cuda") / 10).half()
+        for _ in range(args.warmup):
+            gate_matrix_layer(a, gate, w1, w2, args.topk, True, False)
+        torch.cuda.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for e0, e1 in ev:
+            e0.record()
+            gate_matrix_layer(a, gate, w1, w2, args.topk, True, False)
+            e1.record()
+        torch.cuda.synchronize()
+        t = sorted(e0.elapsed_time(e1) for e0, e1 in ev)[len(ev) // 2] * 1e-3
+        rows.append({"m": m, "us_per_layer": round(t * 1e6, 2), "ref_2mnk_tflops": round(2.0 * m * args.n * args.k / t / 1e12, 3),
+                     "tflops": round(layer_flops(m, args.k, args.n, args.topk) / t / 1e12, 3),
+                     "block": plan(m, args.k, args.n, args.e, args.topk, torch.float16).block})
+    return {"protocol": "fp16, randn/10, n=%d k=%d e=%d topk=%d, gate-matrix layer fused_moe(a, gate, w1, w2, topk, True, False), "
+                        "median of %d event-timed calls" % (args.n, args.k, args.e, args.topk, args.steps),
             "ref_2mnk_tflops_is": "2*m*n*k / t, the figure the reference plots (README moe_bench.png)", "rows": rows}
+
+
+def mfma_stream(torch, N):
+    """The part's sustained rate on a pure MFMA stream (fr_probe_mfma_stream): per MFMA shape, wavefronts per SIMD and
+    operand data; the shader clock from the ratio of the cycle counter to the 100 MHz counter."""
+    lib = N.lib()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.empty(512 * cus, dtype=torch.float32, device="cuda")
+    counts = torch.zeros(2, dtype=torch.int64, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(1)
+    data = {"random bf16 in [1, 2) with random signs": (torch.rand(32768, generator=g, device="cuda") + 1.0) *
+            (torch.randint(0, 2, (32768,), generator=g, device="cuda") * 2 - 1),
+            "zeros": torch.zeros(32768, device="cuda")}
+    rows = []
+    for what, vals in data.items():
+        ops = vals.to(torch.bfloat16).contiguous()
+        for shape in (32, 16):
+            for wps in (1, 2):
+                iters = 3000 * (1 if shape == 32 else 1) // 1
+                per_iter = (16 if wps == 1 else 8) if shape == 32 else (64 if wps == 1 else 32)  # MFMAs per wavefront and iteration
+                best = None
+                for _ in range(3):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    N.check(lib.fr_probe_mfma_stream(shape, wps, iters, ops.data_ptr(), sink.data_ptr(), counts.data_ptr(),
+                                                     torch.cuda.current_stream().cuda_stream))
+                    e1.record()
+                    torch.cuda.synchronize()
+                    ms = e0.elapsed_time(e1)
+                    cyc, ticks = (int(v) for v in counts.cpu())
+                    if best is None or ms < best[0]:
+                        best = (ms, cyc, ticks)
+                ms, cyc, ticks = best
+                mfmas = iters * per_iter                       # per wavefront
+                flop = mfmas * 32768.0 * (1 if shape == 32 else 0.5) * 4 * wps * cus
+                rows.append({"operands": what, "mfma": "32x32x16" if shape == 32 else "16x16x32", "waves_per_simd": wps,
+                             "ms": round(ms, 3), "tflops": round(flop / ms / 1e9, 1),
+                             "shader_clock_ghz": round(cyc / (ticks * 10.0), 3),
+                             "mfma_pipe_busy": round(mfmas * (32 if shape == 32 else 16) * wps / cyc, 3)})
+    return {"metric": "mfma_stream_bf16", "unit": "TFLOP/s", "compute_units": cus, "rows": rows}
+
+
+def vendor_gemm(torch, tokens, shape, steps):
+    """torch.matmul (the vendor's dense GEMM) on the two GEMM shapes of the layer at `tokens` tokens - the same flops,
+    no gather, no SiLU, no routed weight: what a dense kernel sustains on this box next to the grouped ones."""
+    H, F, topk = shape["H"], shape["F"], shape["topk"]
+    g = torch.Generator(device="cuda").manual_seed(3)
+    rows = []
+    for name, (m, n, k) in {"gate/up": (tokens * topk, 2 * F, H), "down": (tokens * topk, H, F)}.items():
+        a = torch.randn(m, k, generator=g, device="cuda").to(torch.bfloat16)
+        b = (torch.randn(n, k, generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+        for _ in range(3):
+            c = a @ b.t()
+        torch.cuda.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for e0, e1 in ev:
+            e0.record()
+            c = a @ b.t()
+            e1.record()
+        torch.cuda.synchronize()
+        t = sorted(e0.elapsed_time(e1) for e0, e1 in ev)[len(ev) // 2] * 1e-3
+        rows.append({"gemm": name, "m": m, "n": n, "k": k, "us": round(t * 1e6, 1), "tflops": round(2.0 * m * n * k / t / 1e12, 1)})
+        del a, b, c
+    return {"metric": "vendor_dense_gemm_bf16", "unit": "TFLOP/s", "tokens": tokens, "rows": rows}
 
 
 def main():
@@ -494,6 +586,12 @@ def main():
     ap.add_argument("-k", type=int, default=4096, help="reference protocol: hidden size")
     ap.add_argument("-e", type=int, default=16, help="reference protocol: experts")
     ap.add_argument("--topk", type=int, default=2, help="reference protocol: experts per token")
+    ap.add_argument("--mfma-stream", action="store_true",
+                    help="only run the pure MFMA stream (fr_probe_mfma_stream): sustained rate and shader clock per MFMA shape")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="only time torch.matmul on the layer's two GEMM shapes at --tokens (dense, no gather): the vendor kernel's rate")
+    ap.add_argument("--prepared", default="", choices=["", "w1", "w2", "both"],
+                    help="run the workloads with weights re-laid-out by prepare_weights (the w2 default of that call, or both)")
     ap.add_argument("--reference-protocol", action="store_true",
                     help="run the reference's sweep (fp16 randn/10, m = 2^0..2^14 at -n -k -e --topk) instead of the workloads")
     args = ap.parse_args()
@@ -505,6 +603,12 @@ def main():
     N.lib()
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
     torch.cuda.set_device(0)
+    if args.mfma_stream:
+        print(json.dumps(mfma_stream(torch, N)))
+        return
+    if args.vendor_gemm:
+        print(json.dumps(vendor_gemm(torch, args.tokens, SHAPES[args.shape], args.steps)))
+        return
     if args.reference_protocol:
         print(json.dumps({"metric": "reference_protocol_moe_bench", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
                           "dtype": "f16", "data": "synthetic", **reference_protocol(torch, N, args)}))
@@ -520,14 +624,18 @@ def main():
         from fast_route_amd import prepare_weights_fp8
         fp8 = prepare_weights_fp8(w1, w2)
         sweep_ms = [16, 256, 4096] if args.shape == "mixtral" else shape["sweep"]
-    head, layer = measure(torch, N, shape, args.tokens, w1, w2, args.steps, args.warmup, args.seed, fp8, flush=flush)
+    prepared = 0
+    if args.prepared and fp8 is None:
+        from fast_route_amd import prepare_weights
+        w1, w2, prepared = prepare_weights(w1, w2, args.prepared)
+    head, layer = measure(torch, N, shape, args.tokens, w1, w2, args.steps, args.warmup, args.seed, fp8, flush=flush, prepared=prepared)
     sweep = []
     if not args.no_sweep:
         for M in sweep_ms:
             if M == args.tokens:
                 sweep.append(head)
                 continue
-            rec, _ = measure(torch, N, shape, M, w1, w2, args.steps, args.warmup, args.seed, fp8, flush=flush)
+            rec, _ = measure(torch, N, shape, M, w1, w2, args.steps, args.warmup, args.seed, fp8, flush=flush, prepared=prepared)
             sweep.append(rec)
     result = {
         "metric": "moe_layer_tflops_%s_%s_M%d" % (args.shape, args.dtype, args.tokens),
@@ -538,7 +646,7 @@ def main():
                                % (args.shape, H, F, E, topk, args.tokens, args.dtype),
                    "tokens": args.tokens, "hidden": H, "ffn": F, "experts": E, "topk": topk, "seed": args.seed,
                    "flops_formula": "6*M*topk*H*F"},
-        "native_library": os.path.basename(N.LIB_PATH),
+        "native_library": os.path.basename(N.LIB_PATH), "weights_prepared": args.prepared or "no",
         "layer_roofline_frac": head["roofline_frac"], "layer_bound": head["bound"],
         "stage_us": head["stage_us"],
         "roofline": kernel_roofline(shape, head, fp8 is not None),

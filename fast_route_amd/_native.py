@@ -56,6 +56,7 @@ SIGNATURES = {
                                  c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_int64, c_void_p]),
     "fr_fused_moe_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int,
                                      c_int, c_int, c_void_p, c_void_p]),
+    "fr_probe_mfma_stream": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "fr_fused_moe": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int,
                              c_int, c_int, c_void_p, c_void_p, c_int64, c_void_p]),
 }

@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libfast_route_hip.so")
-SOURCES = ["fr_error.hip", "gating.hip", "routing.hip", "quant.hip", "moe_gemm.hip", "fused_moe.hip"] + [
+SOURCES = ["fr_error.hip", "gating.hip", "routing.hip", "quant.hip", "moe_gemm.hip", "fused_moe.hip", "probe.hip"] + [
     "moe_gemm_inst_%s_%s.hip" % (t, e) for t in ("bf16", "f16", "fp8") for e in ("silu", "plain", "down")]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -280,6 +280,17 @@ int fr_fused_moe_fp8(const void* x, int x_dtype, const void* w1q, const float* w
                      int64_t F, int E, int topk, int renormalize, void* out, void* workspace,
                      int64_t workspace_bytes, void* stream);
 
+/* ---- measurement aid -------------------------------------------------------
+ * A pure stream of bf16 MFMAs (no loads, no LDS) on every CU: `iters` rounds over 256 accumulator
+ * registers per lane and SIMD, `shape` 32 = v_mfma_f32_32x32x16_bf16, 16 = v_mfma_f32_16x16x32_bf16,
+ * with one or two wavefronts per SIMD.  operands: 65536 bytes of operand bits (random bf16 draw the
+ * power real data draw; zeros do not); sink: 512 floats per CU; counts[2] receives workgroup 0's
+ * elapsed shader-clock cycles and ticks of the 100 MHz counter.  The part lowers its clock under MFMA
+ * load to hold a power budget; this is the ceiling the roofline fractions of the grouped GEMMs are
+ * read against.  No counterpart in the reference. */
+int fr_probe_mfma_stream(int shape, int waves_per_simd, int iters, const void* operands, float* sink,
+                         int64_t* counts, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

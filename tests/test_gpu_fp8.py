@@ -111,6 +111,9 @@ def test_fp8_mixtral_shape_sampled(native):
         ref, _ = oracle.fused_moe_fp8(x[sample].cpu(), w1c, w2c, logits[sample].cpu(), k, True, weights_q=wq)
         o = out[sample].float().cpu()
         assert (o - ref).norm() / ref.norm() <= 1e-2
+        # same quantised operands on both sides: what is left is accumulation order and the bf16 rounding of
+        # the activated row (which can flip an e4m3 code of its re-quantisation) and of the output: the bound of the other fp8 tests
+        assert (o - ref).abs().max() <= 2.0 ** -5 * ref.abs().max(), f"M={M}: max abs err {(o - ref).abs().max():.3e} of {ref.abs().max():.3e}"
         out2 = fused_moe_fp8(x, w1q, w1s, w2q, w2s, logits, k, True)
         assert torch.equal(out, out2)
 
