@@ -60,6 +60,8 @@ struct GemmArgs {
   int num_experts;      // E (persistent form: walk order by expert)
   int long_k;           // down projection (few feature tiles, long K): hint for the 128-row tile's form
   float* tail_ws;       // persistent form only: slice buffers for splitting the last round of tiles along K, or nullptr
+  unsigned x_span;      // bytes of X the tile loads may address (from X in gather mode, from a block's first row otherwise), or 0:
+                        // with it, the loads of padding slots fall outside the buffer resource and fetch nothing
   int add_div;          // EPI_PLAIN: 0 = store row `sorted id` of out; k > 0 = add into row (sorted id / k) of a zero-filled out (packed atomics)
   int w_tiled;          // W is in the prepared layout (see w_byte_offset), not [E, w_rows, K] row-major
   int setup_only;       // do the per-device set-up of the kernel a launch would take (LDS limit, occupancy) and launch nothing
@@ -200,12 +202,16 @@ __device__ __forceinline__ int swizzle(int row, int chunk) {
 // Buffer resource over the whole address space from `p` on.  The pointer is the same in every
 // lane; reading it through the first lane tells the compiler so, which otherwise may keep the
 // resource in vector registers and wrap each load in a loop over the distinct lane values.
+// Byte offset given to the lanes of padding slots when GemmArgs::x_span is set: beyond any span (spans stay below
+// 2 GiB), so the buffer's range check drops the load - no request, no bytes moved; what the LDS then holds for
+// those rows only ever reaches accumulator columns of padding slots, which no epilogue stores as a pair's result.
+constexpr unsigned kSkipOffset = 0x80000000u;
 template <typename T>
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_rsrc(const T* p) {
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_rsrc(const T* p, unsigned num_records = 0xFFFFFFFFu) {
   const uint64_t v = reinterpret_cast<uint64_t>(p);
   const uint64_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(v))));
   const uint64_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint32_t>(v >> 32))));
-  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(hi << 32 | lo), 0, -1, 0x00020000);
+  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(hi << 32 | lo), 0, static_cast<int>(num_records), 0x00020000);
 }
 #endif
 
@@ -560,7 +566,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     // first row; gathered rows and an expert's weights must span less than 4 GiB
     // (checked by the launcher).
     const int64_t xrow0 = a.top_k > 0 ? 0 : static_cast<int64_t>(pid_t) * BT;
-    const __amdgpu_buffer_rsrc_t xrs = uniform_rsrc(X + xrow0 * a.ldx);
+    const __amdgpu_buffer_rsrc_t xrs = uniform_rsrc(X + xrow0 * a.ldx, a.x_span ? a.x_span : 0xFFFFFFFFu);
     const __amdgpu_buffer_rsrc_t wrs = uniform_rsrc(W);
     const bool issuer = wave_u < NW / IW;
     const int wstep = a.w_tiled ? (C::BKB / kTileBytes) * kTilePiece : C::BKB;  // bytes from one K tile of W to the next
@@ -571,6 +577,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
       const int slot = (i * NW + vw) * kWave + lane;
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
       xsrc[ih] = static_cast<unsigned>(((x_src_row(rr) - xrow0) * a.ldx + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));
+      if (a.x_span && a.sorted[pid_t * BT + rr] >= a.num_valid) xsrc[ih] = kSkipOffset;
     }
 #pragma unroll
     for (int ih = 0; ih < WI * IW; ++ih) {
@@ -734,6 +741,13 @@ int launch_gemm(const GemmArgs& a, int splits, hipStream_t st) {
     if (x_rows * a.ldx * es >= lim || w_rows * a.ldw * es >= lim)
       return fail(FR_E_SHAPE, "token rows (%lld x %lld) or one expert's weights (%lld x %lld) span 4 GiB or more",
                   (long long)x_rows, (long long)a.ldx, (long long)w_rows, (long long)a.ldw);
+    if (x_rows * a.ldx * es < (int64_t(1) << 31)) {
+      GemmArgs b = a;
+      b.x_span = static_cast<unsigned>(x_rows * a.ldx * es);
+      const unsigned gx = static_cast<unsigned>(a.num_t_blocks) * static_cast<unsigned>(a.num_f_tiles);
+      hipLaunchKernelGGL((moe_gemm_kernel<T, C, EPI>), dim3(gx, splits), dim3(C::NT), C::LDS_BYTES, st, b);
+      return check_launch("moe_gemm_kernel");
+    }
   }
   const unsigned grid_x = static_cast<unsigned>(a.num_t_blocks) * static_cast<unsigned>(a.num_f_tiles);
   hipLaunchKernelGGL((moe_gemm_kernel<T, C, EPI>), dim3(grid_x, splits), dim3(C::NT), C::LDS_BYTES, st, a);

@@ -250,23 +250,22 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   // ---- address sets: A = tile being multiplied, B = the workgroup's next tile --------
   int pid_t, pid_f, expert, kb, kn, tu;  // current unit: tile, first K tile and K tile count, slice buffer
   int n_pid_t = 0, n_pid_f = 0, n_expert = 0, n_kb = 0, n_kn = 0, n_tu = -1;
-  int n_sid[XI * IW];  // sorted ids of the next tile's load rows (gather mode), fetched a tile ahead
+  int n_sid[XI * IW];  // sorted ids of the next tile's load rows, fetched a tile ahead
   unsigned xsrcA[XI * IW], wsrcA[WI * IW], xsrcB[XI * IW], wsrcB[WI * IW];
   __amdgpu_buffer_rsrc_t xrsA, wrsA, xrsB, wrsB;
 #define FR_MAKE_SET(pt_, pf_, ex_, kb_, SIDOF, xsrc_, wsrc_, xrs_, wrs_)                                     \
   {                                                                                                          \
     const int64_t xrow0_ = a.top_k > 0 ? 0 : static_cast<int64_t>(pt_) * BT;                                 \
     const int64_t kfirst_ = k0 + static_cast<int64_t>(kb_) * BK;                                             \
-    xrs_ = uniform_rsrc(X + xrow0_ * a.ldx);                                                                 \
+    xrs_ = uniform_rsrc(X + xrow0_ * a.ldx, a.x_span ? a.x_span : 0xFFFFFFFFu);                              \
     wrs_ = uniform_rsrc(static_cast<const T*>(a.W) + static_cast<int64_t>(ex_) * a.w_expert_stride);         \
     _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) {                                                 \
       FR_SLOT_ROW(ih, rr, c)                                                                                 \
       int64_t row_ = rr;                                                                                     \
-      if (a.top_k > 0) {                                                                                     \
-        const int sid_ = SIDOF;                                                                              \
-        row_ = sid_ < a.num_valid ? sid_ / a.top_k : 0;                                                      \
-      }                                                                                                      \
+      const int sid_ = SIDOF;                                                                                \
+      if (a.top_k > 0) row_ = sid_ < a.num_valid ? sid_ / a.top_k : 0;                                       \
       xsrc_[ih] = static_cast<unsigned>((row_ * a.ldx + kfirst_ + c * EPC) * static_cast<int64_t>(sizeof(T))); \
+      if (a.x_span && sid_ >= a.num_valid) xsrc_[ih] = kSkipOffset;                                          \
     }                                                                                                        \
     _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) {                                                 \
       FR_SLOT_ROW(ih, rr, c)                                                                                 \
@@ -435,12 +434,10 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     }                                                                                                      \
     if (NEXT) {                                                                                            \
       FR_UNIT(unit + 1, n_pid_t, n_pid_f, n_expert, n_kb, n_kn, n_tu)                                      \
-      if (a.top_k > 0) {                                                                                   \
-        _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) {                                           \
-          FR_SLOT_ROW(ih, rr, c)                                                                           \
-          (void)c;                                                                                         \
-          n_sid[ih] = a.sorted[n_pid_t * BT + rr];                                                         \
-        }                                                                                                  \
+      _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) {                                             \
+        FR_SLOT_ROW(ih, rr, c)                                                                             \
+        (void)c;                                                                                           \
+        n_sid[ih] = a.sorted[n_pid_t * BT + rr];                                                           \
       }                                                                                                    \
     }                                                                                                      \
     _Pragma("unroll") for (int j = 0; j < C::JF; ++j)                                                      \
@@ -662,6 +659,7 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
                 (long long)x_rows, (long long)a.ldx, (long long)w_rows, (long long)a.ldw);
   a.group_t = tunables().group_m ? tunables().group_m : kChunkBlocks;
   if (tunables().no_tail_split) a.tail_ws = nullptr;
+  a.x_span = x_rows * a.ldx * es < (int64_t(1) << 31) ? static_cast<unsigned>(x_rows * a.ldx * es) : 0u;
   int resident = 0;
   const int rc = persistent_grid<T, C, EPI>(&resident);
   if (rc != FR_OK) return rc;
