@@ -227,6 +227,32 @@ def measure(torch, N, shape, M, w1, w2, steps, warmup, seed, fp8=None, flush=Fal
     return rec, layer
 
 
+def graph_replay_us(torch, layer, reps=20, per_graph=8):
+    """Median time of one layer pass when `per_graph` passes are captured into one HIP graph and the graph
+    is replayed: what a serving loop that captures its launch-bound steps pays per layer.  The fused entry
+    point launches kernels only (no allocation, no memset node), so it is captured as it is."""
+    layer.fused()  # first call outside the capture: set-up of the kernels' attributes
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    keep = layer.stream
+    with torch.cuda.stream(side):
+        layer.stream = side.cuda_stream
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(per_graph):
+                layer.fused()
+        layer.stream = keep
+    ref = layer.out.clone()
+    times = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(); graph.replay(); b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b) * 1e3 / per_graph)
+    assert torch.equal(layer.out, ref), "graph replay changed the layer's output"
+    return round(sorted(times)[len(times) // 2], 2)
+
+
 def kernel_roofline(shape, rec, fp8=False):
     """Roofline of the dominant kernel (gate/up grouped GEMM + SiLU*mul) from its
     event-measured average duration."""
@@ -328,8 +354,9 @@ def cpu_baseline(torch, shape, layer, sample_tokens):
             "ref_max_abs": ref.abs().max().item()}
 
 
-def oracle_error(torch, shape, layer, tokens=48, fp8=None):
-    """Max-abs error of the layer's last output against the CPU oracle on an evenly spaced sample of tokens."""
+def oracle_error(torch, shape, layer, tokens=48, fp8=None, plain=None):
+    """Max-abs error of the layer's last output against the CPU oracle on an evenly spaced sample of tokens.
+    plain: (w1, w2) as the reference lays them out, when the layer holds prepared (re-laid-out) weights."""
     import oracle
     layer.fused()
     torch.cuda.synchronize()
@@ -345,7 +372,8 @@ def oracle_error(torch, shape, layer, tokens=48, fp8=None):
               w2q.cpu().numpy().reshape(E * w2q.shape[1], w2q.shape[2]), w2s.cpu().numpy().reshape(-1))
         ref, _ = oracle.fused_moe_fp8(x, layer.w1.cpu(), layer.w2.cpu(), logits, shape["topk"], True, weights_q=wq)
     else:
-        ref = oracle.fused_moe(x, layer.w1.cpu(), layer.w2.cpu(), logits, shape["topk"], True)
+        pw1, pw2 = plain if plain is not None else (layer.w1, layer.w2)
+        ref = oracle.fused_moe(x, pw1.cpu(), pw2.cpu(), logits, shape["topk"], True)
     got = layer.out[idx.cuda()].float().cpu()
     return {"tokens_checked": int(idx.numel()), "max_abs_err": (got - ref).abs().max().item(),
             "ref_max_abs": ref.abs().max().item(),
@@ -424,9 +452,12 @@ def other_configs(torch, N, args, mixtral_weights):
     shape = SHAPES["small"]
     w1, w2 = make_weights(torch, shape, args.seed)
     rec, layer = measure(torch, N, shape, 64, w1, w2, steps, warmup, args.seed, flush=True)
-    warm, _ = measure(torch, N, shape, 64, w1, w2, steps, warmup, args.seed)
+    warm, wlayer = measure(torch, N, shape, 64, w1, w2, steps, warmup, args.seed)
     out["small"] = dict(compact(rec), stage_us=rec["stage_us"], cache_flush=rec["cache_flush"],
-                        us_per_layer_back_to_back=warm["us_per_layer"], vs_oracle=oracle_error(torch, shape, layer, 64))
+                        us_per_layer_back_to_back=warm["us_per_layer"],
+                        us_per_layer_graph_replay=graph_replay_us(torch, wlayer),
+                        vs_oracle=oracle_error(torch, shape, layer, 64))
+    del wlayer
     del w1, w2, layer
     # routing-only stress: gating + block-aligned sort, bit-exact against the oracle
     out["routing_stress"] = {"tokens": 65536, "experts": 64, "topk": 6, "bound": "hbm (latency bound in practice)",
@@ -438,6 +469,8 @@ def other_configs(torch, N, args, mixtral_weights):
     for M in shape["sweep"]:
         rec, layer = measure(torch, N, shape, M, w1, w2, steps, warmup, args.seed)
         sweep.append(dict(compact(rec), stage_us=rec["stage_us"]))
+        if M == 1:  # four launches of a few microseconds each: the launch-bound end
+            sweep[-1]["us_per_layer_graph_replay"] = graph_replay_us(torch, layer)
     out["fine"] = {"workload": "H=2048 F=1408 E=64 top-6, Zipf(1.2)-skewed load, bf16", "sweep": sweep,
                    "vs_oracle_M8192": oracle_error(torch, shape, layer)}
     del w1, w2, layer
@@ -462,7 +495,7 @@ def other_configs(torch, N, args, mixtral_weights):
         rec, layer = measure(torch, N, shape, M, w1, w2p, steps, warmup, args.seed, prepared=flags)
         sweep.append(dict(compact(rec), stage_us=rec["stage_us"]))
     out["prepared_w2"] = {"workload": "Mixtral shape bf16, w2 re-laid-out once by prepare_weights (64-row x 128-byte tiles); w1 as the reference has it",
-                          "sweep": sweep, "vs_oracle_M16384": oracle_error(torch, shape, layer)}
+                          "sweep": sweep, "vs_oracle_M16384": oracle_error(torch, shape, layer, plain=(w1, w2))}
     del w2p, layer
     return out
 

@@ -56,7 +56,7 @@ def test_host_only_calls_need_no_gpu():
 def test_plan_table():
     """The tile plan is host logic: routing block and K slices of the down projection per token count,
     as documented (Mixtral shape: 16-row blocks up to 8 pairs per expert, 32 below 26, 64 below 52 at
-    H >= 4096, 128 below 368, 256 above; the fine-grained shape with H = 2048 has no 64-row range and
+    H >= 4096, 128 below 560, 256 above; the fine-grained shape with H = 2048 has no 64-row range and
     switches to 256 rows at 640 pairs per expert)."""
     from fast_route_amd import _native
     lib = _native.lib()
@@ -68,7 +68,7 @@ def test_plan_table():
         return p.block, p.split_k
 
     mix = lambda M, dt=_native.FR_BF16: plan(M, 4096, 14336, 8, 2, dt)
-    assert [mix(M)[0] for M in (1, 32, 33, 103, 104, 207, 208, 1471, 1472)] == [16, 16, 32, 32, 64, 64, 128, 128, 256]
+    assert [mix(M)[0] for M in (1, 32, 33, 103, 104, 207, 208, 2239, 2240)] == [16, 16, 32, 32, 64, 64, 128, 128, 256]
     assert mix(1) == (16, 4) and mix(2) == (16, 2) and mix(3) == (16, 4) and mix(4) == (16, 4) and mix(16) == (16, 1)
     assert mix(128) == (64, 2)
     assert mix(4096)[1] == 1 and plan(4096, 4096, 14336, 8, 2)[0] == 256
