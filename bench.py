@@ -282,6 +282,14 @@ def kernel_roofline(shape, rec, fp8=False):
             "avg_launch_us": round(dur * 1e6, 2), "algorithmic_bytes_per_launch": byts}
 
 
+def tunables_now(N):
+    """The library's study knobs at the time of the run (all zero = every choice left to the plan)."""
+    import ctypes
+    t = N.FrMoeTunables()
+    N.check(N.lib().fr_moe_get_tunables(ctypes.byref(t)))
+    return {name: int(getattr(t, name)) for name, _ in t._fields_}
+
+
 def kernel_sources_sha():
     """Hash of the HIP sources the library is built from: ties an offline counter record to the kernels it measured."""
     root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fast_route_amd", "csrc")
@@ -680,6 +688,7 @@ def main():
                    "tokens": args.tokens, "hidden": H, "ffn": F, "experts": E, "topk": topk, "seed": args.seed,
                    "flops_formula": "6*M*topk*H*F"},
         "native_library": os.path.basename(N.LIB_PATH), "weights_prepared": args.prepared or "no",
+        "tunables": tunables_now(N),
         "layer_roofline_frac": head["roofline_frac"], "layer_bound": head["bound"],
         "stage_us": head["stage_us"],
         "roofline": kernel_roofline(shape, head, fp8 is not None),

@@ -169,6 +169,12 @@ int fr_moe_prepare(int dtype);
  *              16384 tokens, 149 against 146 us at 16 tokens)
  * fr_moe_get_plan, fr_fused_moe, fr_fused_experts, fr_fused_moe_fp8 and the staged GEMM entry
  * points all see them.  fr_moe_set_tunables(NULL) restores the defaults.
+ * The staged entry points read the knobs when they are called, not when the plan was made: a
+ * caller that sized `partial` / `tail_ws` from a plan, changed the knobs and then calls the staged
+ * GEMMs runs the old sizes with the new group_m / no_tail_split (never out of bounds: `block` and
+ * `split_k` are the call's own arguments, and the slices actually run are min(split_k, what K
+ * allows at 8 K tiles per slice)).  A study should take a new plan after every change and record
+ * fr_moe_get_tunables() next to its timings, as bench.py does.
  * Replaces: the per-GEMM config dictionaries edited by hand in the reference's tile study
  * (block_m / group_m / split_k; block_n and block_k are fixed per block size on this hardware),
  * fast_route/benchmarks/swizzle_moe/v1_moe_fused.py:311-344. */
