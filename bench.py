@@ -290,22 +290,26 @@ def tunables_now(N):
     return {name: int(getattr(t, name)) for name, _ in t._fields_}
 
 
+GEMM_KERNEL_SOURCES = ("moe_gemm_kernel.h", "moe_gemm_persistent.h", "moe_gemm_tiles.h", "moe_gemv.h", "moe_gemm.hip")
+
+
 def kernel_sources_sha():
-    """Hash of the HIP sources the library is built from: ties an offline counter record to the kernels it measured."""
+    """Hash of the sources of the grouped-GEMM kernels (tile kernels, their persistent form, the tile table and
+    dispatch, the weight-row kernels): ties an offline counter record to the kernels it measured."""
     root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fast_route_amd", "csrc")
     h = hashlib.sha256()
-    for name in sorted(os.listdir(root)):
-        if name.endswith((".h", ".hip")):
-            with open(os.path.join(root, name), "rb") as f:
-                h.update(name.encode() + b"\0" + f.read())
+    for name in GEMM_KERNEL_SOURCES:
+        with open(os.path.join(root, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read())
     return h.hexdigest()[:16]
 
 
-def recorded_traffic(metric):
+def recorded_traffic(metric, block):
     """HBM bytes per launch of the dominant kernel for this workload, as measured offline with
     rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE runs, scaled by the copy probe) and recorded
-    in profiles/hbm_traffic.json; None when the workload has no record or the record was taken
-    with other kernel sources than the ones present."""
+    in profiles/hbm_traffic.json; None when the workload has no record, when the record was taken
+    with other GEMM kernel sources than the ones present, or when the plan now picks another
+    routing block (i.e. another tile) for this workload than the one that was measured."""
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
     try:
         with open(path) as f:
@@ -313,7 +317,7 @@ def recorded_traffic(metric):
     except (OSError, ValueError):
         return None
     rec = doc.get(metric)
-    if not rec or doc.get("kernel_sources_sha") != kernel_sources_sha():
+    if not rec or doc.get("kernel_sources_sha") != kernel_sources_sha() or rec.get("block") != block:
         return None
     return rec["traffic_bytes"]
 
@@ -694,7 +698,7 @@ def main():
         "roofline": kernel_roofline(shape, head, fp8 is not None),
         "sweep": sweep,
     }
-    result["roofline"]["traffic"] = recorded_traffic(result["metric"])
+    result["roofline"]["traffic"] = recorded_traffic(result["metric"], head["block"])
     if args.copy_probe:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
         dst = torch.empty_like(src)

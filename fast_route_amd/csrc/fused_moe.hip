@@ -108,8 +108,9 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // The 256-row tile's advantage grows with the K of the gate/up GEMM (its start-up per
   // tile is amortised over more K tiles); measured crossovers: 512..640 pairs per expert
   // at H = 4096 (F = 14336, E = 8: 2048 tokens 1380 us with 128 rows against 1435 with 256, 2560 tokens
-  // 1810 against 1662), 576..768 at H = 2048 (F = 1408, E = 64).
-  const double t256 = H >= 4096 ? 560.0 : (H <= 2048 ? 640.0 : 640.0 - (H - 2048) * (80.0 / 2048.0));
+  // 1810 against 1662).  At H = 2048 (F = 1408, E = 64, top-6: 32 and 22 K tiles per output tile) the 128-row
+  // tile stays ahead as far as measured: 768 / 1536 pairs per expert 960 / 1738 us against 1002 / 1776.
+  const double t256 = H >= 4096 ? 560.0 : (H <= 2048 ? 4096.0 : 4096.0 - (H - 2048) * (3536.0 / 2048.0));
   // Between 26 and 52 pairs per expert with a long gate/up K the 64-row tile wins: one block per expert
   // where 32-row blocks stream every expert's weights through the CUs twice, and half the MFMA and LDS work
   // of the 128-row tile (measured at H = 4096, F = 14336, E = 8: M = 112..192 4-6 % faster than either;

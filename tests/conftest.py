@@ -17,3 +17,12 @@ def native():
     """The loaded C-ABI library; GPU tests fail loudly when it is not built."""
     from fast_route_amd import _native
     return _native.lib()
+
+
+@pytest.fixture
+def rows256():
+    """256-row routing blocks for the duration of a test: the plan keeps shapes with a short gate/up K on
+    128-row blocks, and the tests of the 256-row tiles' last-round split build their routing for 256."""
+    import fast_route_amd as fr
+    with fr.tunables(block=256):
+        yield

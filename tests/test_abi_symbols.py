@@ -57,7 +57,7 @@ def test_plan_table():
     """The tile plan is host logic: routing block and K slices of the down projection per token count,
     as documented (Mixtral shape: 16-row blocks up to 8 pairs per expert, 32 below 26, 64 below 52 at
     H >= 4096, 128 below 560, 256 above; the fine-grained shape with H = 2048 has no 64-row range and
-    switches to 256 rows at 640 pairs per expert)."""
+    keeps 128 rows up to 4096 pairs per expert)."""
     from fast_route_amd import _native
     lib = _native.lib()
 
@@ -74,7 +74,7 @@ def test_plan_table():
     assert mix(4096)[1] == 1 and plan(4096, 4096, 14336, 8, 2)[0] == 256
     assert [mix(M, _native.FR_FP8_E4M3)[0] for M in (103, 104, 207, 208)] == [32, 64, 64, 128]
     fine = lambda M: plan(M, 2048, 1408, 64, 6)[0]
-    assert [fine(M) for M in (85, 86, 341, 342, 6826, 6827)] == [16, 32, 32, 128, 128, 256]
+    assert [fine(M) for M in (85, 86, 341, 342, 43690, 43691)] == [16, 32, 32, 128, 128, 256]
     # the scratch for splitting the last round exists exactly for 128- and 256-row blocks with a long K
     p = _native.FrMoePlan()
     lib.fr_moe_get_plan(4096, 4096, 14336, 8, 2, _native.FR_BF16, p)

@@ -118,7 +118,7 @@ def test_fp8_mixtral_shape_sampled(native):
         assert torch.equal(out, out2)
 
 
-def test_fp8_down_projection_tail_split(native):
+def test_fp8_down_projection_tail_split(native, rows256):
     """Routing built so that the down projection has 8 token blocks x 2 feature tiles of 256 rows
     over K = 4096: two tiles per XCD, each cut into 8 K slices whose sum the fix-up kernel scales
     (activation-row scale x weight-row scale x routed weight) and rounds."""

@@ -221,7 +221,7 @@ def test_block_256_several_tiles_per_workgroup(native, dtype):
 
 
 @pytest.mark.parametrize("case", ["gate_up_after_whole_tile", "down_first_unit", "with_and_without_scratch"])
-def test_last_round_of_tiles_split_along_k(native, case):
+def test_last_round_of_tiles_split_along_k(native, rows256, case):
     """256-row tiles that only partly fill the last round of workgroups are cut along K over
     the idle ones and summed by a second launch.  Routing is constructed so that the tile
     counts are exact (k = 1, every expert a whole number of 256-token blocks):

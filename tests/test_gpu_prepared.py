@@ -16,6 +16,10 @@ def _say(msg):
     sys.stdout.flush()
 
 
+def ref_scale(t):
+    return t.float().abs().max().cpu()
+
+
 def _inputs(M, H, Fd, E, seed, dtype, zipf=False):
     x, logits, w1, w2 = oracle.make_inputs(M, H, Fd, E, seed=seed, zipf=zipf)
     return x.to(dtype), logits, w1.to(dtype), w2.to(dtype)
@@ -73,6 +77,14 @@ def test_layer_with_prepared_weights(native, M, dtype, which):
     torch.cuda.synchronize()
     if M > 4:  # same kernels, same order of every sum
         assert torch.equal(out_p, out_r), f"M={M}: prepared and row-major outputs differ"
+    if M == 3000:  # the plan keeps this width on 128-row blocks: the 256-row tiles (32x32x16 MFMA form) by override
+        import fast_route_amd as fr
+        with fr.tunables(block=256):
+            out_p2 = fused_moe(xd, w1p, w2p, ld, 2, True, weights_prepared=flags)
+            out_r2 = fused_moe(xd, w1d, w2d, ld, 2, True)
+            torch.cuda.synchronize()
+        assert torch.equal(out_p2, out_r2), "256-row blocks: prepared and row-major outputs differ"
+        assert (out_p2.float() - out_p.float()).abs().max().cpu() <= 2.0 ** -6 * ref_scale(out_p)
     ref = oracle.fused_moe(x, w1, w2, logits, 2, True)
     err = (out_p.float().cpu() - ref).abs().max()
     assert err <= 2.0 ** -6 * ref.abs().max(), f"M={M}: max abs err {err:.3e}"
@@ -115,7 +127,7 @@ def test_mixtral_width_with_prepared_weights(native):
     w1 = (torch.randn(E, 2 * Fd, H, generator=g) * 0.02).to(torch.bfloat16).cuda()
     w2 = (torch.randn(E, H, Fd, generator=g) * 0.02).to(torch.bfloat16).cuda()
     w1p, w2p, flags = prepare_weights(w1, w2, "both")
-    for M in (6, 20, 40, 150, 520):
+    for M in (6, 20, 40, 150, 520, 600):  # 600: 256-row blocks (16x16x32 form)
         _say(f"prepared Mixtral width M={M}")
         x = torch.randn(M, H, generator=g).to(torch.bfloat16).cuda()
         logits = torch.randn(M, E, generator=g).cuda()
