@@ -1,6 +1,7 @@
 // Composite entry points: tile plan, workspace carving, and the whole layer as
 // one sequence of launches on the caller's stream.
 #include "fr_common.h"
+#include <cmath>
 
 namespace fr {
 namespace {
@@ -79,8 +80,8 @@ extern "C" int fr_moe_set_tunables(const fr_moe_tunables* t) {
     g_tunables = fr_moe_tunables{0, 0, 0, 0, 0};
     return FR_OK;
   }
-  FR_REQUIRE(t->block == 0 || t->block == 16 || t->block == 32 || t->block == 64 || t->block == 128 || t->block == 256,
-             FR_E_SHAPE, "fr_moe_set_tunables: block=%d not in {0, 16, 32, 64, 128, 256}", t->block);
+  FR_REQUIRE(t->block == 0 || t->block == 16 || t->block == 32 || t->block == 64 || t->block == 128 || t->block == 160 || t->block == 256,
+             FR_E_SHAPE, "fr_moe_set_tunables: block=%d not in {0, 16, 32, 64, 128, 160, 256}", t->block);
   FR_REQUIRE(t->split_k >= 0 && t->split_k <= 64, FR_E_SHAPE, "fr_moe_set_tunables: split_k=%d outside [0, 64]", t->split_k);
   FR_REQUIRE(t->group_m >= 0 && t->group_m <= 64, FR_E_SHAPE, "fr_moe_set_tunables: group_m=%d outside [0, 64]", t->group_m);
   FR_REQUIRE(t->no_tail_split == 0 || t->no_tail_split == 1, FR_E_SHAPE, "fr_moe_set_tunables: no_tail_split=%d", t->no_tail_split);
@@ -121,6 +122,34 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   else if (avg < 52 && H >= 4096) block = 64;
   else if (avg < t256) block = 128;
   else block = 256;
+  // 160-row blocks (2-byte operands, a gate/up K of at least 32 K tiles): the same three-slot ring as the 128-row
+  // tile with a quarter more rows per pass of an expert's weights through LDS.  Under uniform routing an expert
+  // gets avg +- sqrt(avg) pairs, so with avg = 128, 256, 384, 512 every other expert needs one 128-row block more
+  // than avg / 128; 160 rows absorb the spread.  Taken where the expected number of blocks per expert drops by a
+  // tenth or more, or the expected rows the MFMAs multiply (whole half-blocks: a wavefront row is skipped when
+  // all its rows are padding) by 2 %; measured on 8 experts, H = 4096, 128 / 160 / 256 rows:
+  //   tokens  512  681 / 618         us      1536  1143 / 1112 / 1132       3072        1906 / 1939
+  //           640  753 / 749                 1792  1236 / 1179 / 1192       4096        2433 / 2485
+  //           768  715 / 743 (128 stays)     2048  1393 / 1386 / 1441       5120        2988 / 2975
+  //           896  828 / 770                 2560  1706 / 1623 / 1685       6144        3507 / 3478
+  //          1024  874 / 801                                                8192        4658 / 4512
+  // With a 160-row candidate the 256-row tile takes over at 1200 pairs per expert (H >= 4096).  Below 112 pairs per expert one
+  // block holds an expert either way and the smaller tile is cheaper (256 / 384 tokens: 548 / 556, 580 / 602 us);
+  // with H = 1024 (16 K tiles) the 160-row tile loses (700 tokens: 85 / 96 us).
+  if ((block == 128 || block == 256) && (dtype == FR_BF16 || dtype == FR_F16) && H >= 2048 && E <= 1022 && avg >= 112 &&
+      avg < (H >= 4096 ? 1200.0 : t256)) {
+    const double sigma = sqrt(avg * (1.0 - 1.0 / E)) + 1e-9;
+    auto tail = [&](double x) { return 0.5 * erfc((x - avg) / (sigma * 1.4142135623730951)); };  // P(pairs of an expert > x)
+    auto expected = [&](int rows) {  // expected multiples of `rows` that hold an expert's pairs
+      double sum = 1.0;
+      for (int k = 1; k * rows < avg + 8 * sigma; ++k) sum += tail(static_cast<double>(k) * rows);
+      return sum;
+    };
+    const double b128 = expected(128), b160 = expected(160);
+    const double c128 = expected(64) * 64, c160 = expected(80) * 80;
+    const bool take160 = b160 * 1.1 < b128 || c160 <= 0.98 * c128;
+    if (take160) block = 160;
+  }
   if (g_tunables.block) block = g_tunables.block;
   // Down projection: N = H gives few feature tiles, so K is split.
   const int bf = block == 16 ? 64 : (block == 32 ? 128 : 256);

@@ -119,7 +119,7 @@ int64_t tail_scratch_bytes(int block, int dtype, int64_t K, int64_t N, bool gate
   static_assert(Tiles<fp8_t>::T256::BF == C::BF && Tiles<fp8_t>::T256::BKB == C::BKB, "same K tile and feature tile");
   const bool two_byte = dtype == FR_BF16 || dtype == FR_F16;
   if (!two_byte && dtype != FR_FP8_E4M3) return 0;
-  if (!((block == 256 && (two_byte || !gateup)) || block == 128)) return 0;
+  if (!((block == 256 && (two_byte || !gateup)) || block == 128 || (block == 160 && two_byte))) return 0;
   const int64_t bk = C::BKB / elem_bytes(dtype), cols = gateup ? C::BF / 2 : C::BF;
   if (K / bk < kTailMinTiles || N % cols != 0) return 0;
   return static_cast<int64_t>(kTailUnits) * C::BT * C::BF * 4;  // sized for the larger tile
@@ -133,7 +133,7 @@ int gateup_impl(const void* x, const float* x_scale, const void* w1, const float
   FR_REQUIRE(!w_tiled || (F % kTileRows == 0 && (H * elem_bytes(dtype)) % kTileBytes == 0), FR_E_SHAPE,
              "%s: prepared weights need F %% %d == 0 and whole %d-byte K tiles", who, kTileRows, kTileBytes);
   FR_REQUIRE(x && w1 && act && sorted && expert_ids && npost, FR_E_NULL, "%s: null pointer", who);
-  FR_REQUIRE(valid_block(block), FR_E_SHAPE, "%s: block=%d not in {16,32,64,128,256}", who, block);
+  FR_REQUIRE(valid_block(block), FR_E_SHAPE, "%s: block=%d not in {16,32,64,128,160,256}", who, block);
   FR_REQUIRE(H > 0 && H % k_multiple(dtype, block) == 0, FR_E_SHAPE, "%s: H=%lld must be a multiple of %d for block %d", who, (long long)H, k_multiple(dtype, block), block);
   FR_REQUIRE(F > 0 && F % 8 == 0, FR_E_SHAPE, "%s: F=%lld must be a positive multiple of 8", who, (long long)F);
   FR_REQUIRE(topk >= 1 && E >= 1 && M * topk < (int64_t(1) << 30), FR_E_SHAPE, "%s: M*topk too large", who);
@@ -188,7 +188,7 @@ int down_impl(const void* act, const float* act_scale, const void* w2, const flo
   FR_REQUIRE(!w_tiled || (H % kTileRows == 0 && (F * elem_bytes(dtype)) % kTileBytes == 0), FR_E_SHAPE,
              "%s: prepared weights need H %% %d == 0 and whole %d-byte K tiles", who, kTileRows, kTileBytes);
   FR_REQUIRE(act && w2 && topk_weights && partial && out && sorted && expert_ids && npost, FR_E_NULL, "%s: null pointer", who);
-  FR_REQUIRE(valid_block(block), FR_E_SHAPE, "%s: block=%d not in {16,32,64,128,256}", who, block);
+  FR_REQUIRE(valid_block(block), FR_E_SHAPE, "%s: block=%d not in {16,32,64,128,160,256}", who, block);
   FR_REQUIRE(F > 0 && F % k_multiple(dtype, block) == 0, FR_E_SHAPE, "%s: F=%lld must be a multiple of %d for block %d", who, (long long)F, k_multiple(dtype, block), block);
   FR_REQUIRE(H > 0 && H % 4 == 0, FR_E_SHAPE, "%s: H=%lld must be a positive multiple of 4", who, (long long)H);
   FR_REQUIRE(split_k >= 1 && split_k <= 64, FR_E_SHAPE, "%s: split_k=%d outside [1, 64]", who, split_k);
@@ -287,7 +287,7 @@ extern "C" int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, vo
   FR_REQUIRE(A && B && C && sorted_token_ids && expert_ids && num_tokens_post_pad, FR_E_NULL, "fr_moe_grouped_gemm: null pointer");
   FR_REQUIRE(!mul_routed_weight || topk_weights, FR_E_NULL, "fr_moe_grouped_gemm: mul_routed_weight without topk_weights");
   FR_REQUIRE(dtype == FR_F16 || dtype == FR_BF16, FR_E_DTYPE, "fr_moe_grouped_gemm: dtype %d not in {f16, bf16}", dtype);
-  FR_REQUIRE(valid_block(block), FR_E_SHAPE, "fr_moe_grouped_gemm: block=%d not in {16,32,64,128,256}", block);
+  FR_REQUIRE(valid_block(block), FR_E_SHAPE, "fr_moe_grouped_gemm: block=%d not in {16,32,64,128,160,256}", block);
   FR_REQUIRE(K > 0 && K % k_multiple(dtype, block) == 0, FR_E_SHAPE, "fr_moe_grouped_gemm: K=%lld must be a positive multiple of %d for block %d", (long long)K, k_multiple(dtype, block), block);
   FR_REQUIRE(N > 0 && N % 4 == 0, FR_E_SHAPE, "fr_moe_grouped_gemm: N=%lld must be a positive multiple of 4", (long long)N);
   FR_REQUIRE(top_k >= 1 && E >= 1, FR_E_SHAPE, "fr_moe_grouped_gemm: top_k=%d E=%d", top_k, E);

@@ -178,12 +178,15 @@ struct Cfg {
   static constexpr int KGROUPS = 64 / TILE;        // lane groups along K in one MFMA
   static constexpr int XCH = BT * CPR, WCH = BF * CPR;
   static constexpr int XL = (XCH + NT - 1) / NT, WL = (WCH + NT - 1) / NT;
-  static constexpr int XI = XCH / (kWave * NW), WI = WCH / (kWave * NW);  // direct-to-LDS loads per wave per tile
+  // direct-to-LDS loads per ISSUING wavefront and tile (an issuing wavefront issues for IW wavefronts: load ih covers
+  // the 64 chunks of virtual wavefront (wave + (ih % IW) * NW / IW) in group ih / IW of NW * 64 chunks; with an odd
+  // count - the 160-row token tile with IW = 2 - the last group is half a group, all of it virtual wavefronts 0..NW/IW-1)
+  static constexpr int XIW = XCH * IW / (kWave * NW), WIW = WCH * IW / (kWave * NW);
   static constexpr int LDS_BYTES = (STAGES_ == 0 ? 2 : STAGES_) * (BT + BF) * BKB;
   static_assert(TT % TILE == 0 && TF % TILE == 0, "wave tile must be a multiple of the MFMA tile");
   static_assert(NT % CPR == 0, "threads must cover whole rows");
-  static_assert(STAGES_ == 0 || (STAGES_ >= 2 && XCH % (kWave * NW) == 0 && WCH % (kWave * NW) == 0),
-                "direct-to-LDS tiles must split evenly over the wavefronts");
+  static_assert(STAGES_ == 0 || (STAGES_ >= 2 && (XCH * IW) % (kWave * NW) == 0 && (WCH * IW) % (kWave * NW) == 0),
+                "direct-to-LDS tiles must split evenly over the issuing wavefronts");
 };
 
 // LDS is 64 banks x 4 B: a 16-lane phase of ds_read_b128 is conflict-free when its
@@ -546,12 +549,12 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     // slots (slot = row*CPR + physical chunk), lane L the L-th of them, so each
     // lane fetches the logical chunk that the swizzle maps to its slot.
     typedef __attribute__((address_space(3))) void* lptr_t;
-    constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, NL = XI + WI;
+    constexpr int S = C::STAGES, NW = C::NW, XIW = C::XIW, WIW = C::WIW;
     // The NL loads that refill a slot are issued in PARTS groups of PER, one group per K-step.
     constexpr int PARTS = C::SPREAD < 1 ? 1 : (C::SPREAD > KS ? KS : C::SPREAD);
     // With IW == 2 the loads of wavefront w + NW/2 are issued by wavefront w: the two share a SIMD, so while
     // one sits in the load issue stage the other keeps the MFMA pipe busy instead of both stalling together.
-    constexpr int IW = C::IW, NLI = NL * IW;  // loads per issuing wavefront per tile
+    constexpr int IW = C::IW, NLI = XIW + WIW;  // loads per issuing wavefront per tile
     constexpr int PER = (NLI + PARTS - 1) / PARTS, P0 = PER < NLI ? PER : NLI;
     static_assert(IW >= 1 && NW % IW == 0, "issue width");
     static_assert(KS % 2 == 0, "fragment double buffering needs an even number of K-steps per tile");
@@ -570,17 +573,18 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
     const __amdgpu_buffer_rsrc_t wrs = uniform_rsrc(W);
     const bool issuer = wave_u < NW / IW;
     const int wstep = a.w_tiled ? (C::BKB / kTileBytes) * kTilePiece : C::BKB;  // bytes from one K tile of W to the next
-    unsigned xsrc[XI * IW], wsrc[WI * IW];  // byte offsets, [load][virtual wavefront]
+    unsigned xsrc[XIW], wsrc[WIW];  // byte offsets, [load][virtual wavefront]
 #pragma unroll
-    for (int ih = 0; ih < XI * IW; ++ih) {
+    for (int ih = 0; ih < XIW; ++ih) {
       const int i = ih / IW, vw = (wave_u + (ih % IW) * (NW / IW)) % NW;
       const int slot = (i * NW + vw) * kWave + lane;
-      const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
+      // (with an odd load count the last index lies beyond the tile for the wavefronts that issue nothing: clamped)
+      const int rr = min(slot / CPR, BT - 1), c = swizzle<CPR>(rr, slot % CPR);
       xsrc[ih] = static_cast<unsigned>(((x_src_row(rr) - xrow0) * a.ldx + k0 + c * EPC) * static_cast<int64_t>(sizeof(T)));
       if (a.x_span && a.sorted[pid_t * BT + rr] >= a.num_valid) xsrc[ih] = kSkipOffset;
     }
 #pragma unroll
-    for (int ih = 0; ih < WI * IW; ++ih) {
+    for (int ih = 0; ih < WIW; ++ih) {
       const int i = ih / IW, vw = (wave_u + (ih % IW) * (NW / IW)) % NW;
       const int slot = (i * NW + vw) * kWave + lane;
       const int rr = slot / CPR, c = swizzle<CPR>(rr, slot % CPR);
@@ -593,14 +597,14 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_kernel(const GemmArgs
 #define FR_ISSUE_ONE(tile_, slot_, q_)                                                                     \
   {                                                                                                        \
     const int vw_ = wave_u + ((q_) % IW) * (NW / IW);                                                      \
-    if ((q_) < WI * IW) {                                                                                  \
+    if ((q_) < WIW) {                                                                                  \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
           wrs, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vw_) * (kWave * 16)), \
-          16, wsrc[(q_) < WI * IW ? (q_) : 0], (tile_) * wstep, 0, FR_W_AUX);                                    \
+          16, wsrc[(q_) < WIW ? (q_) : 0], (tile_) * wstep, 0, FR_W_AUX);                                    \
     } else {                                                                                               \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
-          xrs, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WI * IW) / IW) * NW + vw_) * (kWave * 16)), \
-          16, xsrc[(q_) < WI * IW ? 0 : (q_) - WI * IW], (tile_) * C::BKB, 0, 0);                          \
+          xrs, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WIW) / IW) * NW + vw_) * (kWave * 16)), \
+          16, xsrc[(q_) < WIW ? 0 : (q_) - WIW], (tile_) * C::BKB, 0, 0);                          \
     }                                                                                                      \
   }
 #define FR_ISSUE_PART(tile_, slot_, p_)                                                                    \

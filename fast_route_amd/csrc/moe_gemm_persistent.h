@@ -78,13 +78,13 @@ __device__ __forceinline__ int xcd_round_tile(const XcdSchedule& s, int nper, in
 // hold at any moment - then share one expert's weight tiles and a few token blocks, and a weight
 // tile is fetched by one chunk only (groups of a fixed number of blocks straddle experts and fetch
 // two experts' tiles each: measured 4.6 GB through L2 per launch against 2.1 GB of operands).
-constexpr int kMaxExperts = 1024;  // limit of the routing entry points
+constexpr int kWalkTable = 1024;   // ints of LDS for the walk table: with the 160-row tile's ring (159744 bytes) exactly the 160 KB of a CU
+constexpr int kMaxExperts = kWalkTable - 2;  // experts the persistent form takes (the routing entry points take 1024: those launches run the plain kernel)
 constexpr int kChunkBlocks = 8;    // token blocks per chunk, at most (measured 4 / 8 / 16: 1675 / 1648 / 1640 us at M=4096,
                                    // 8 and 12 best at M=16384)
 // off[e] = first token block of expert e among the nt real blocks, off[E] = nt; off[kMaxExperts + 1] = 1
 // if expert_ids does not ascend (routing arrays of another producer, legal for the op-level GEMM): then
 // every tile takes the plain row-major walk, since the table describes no partition of the blocks.
-constexpr int kWalkTable = kMaxExperts + 2;
 __device__ __forceinline__ void expert_block_offsets(const GemmArgs& a, int nt, int* off, int tid, int nthreads) {
   if (tid == 0) off[kMaxExperts + 1] = 0;
   for (int e = tid; e <= a.num_experts; e += nthreads) {
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   constexpr int BK = C::BKB / static_cast<int>(sizeof(T));
   constexpr int KS = CPR / (C::KGROUPS * FC);
   constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
-  constexpr int S = C::STAGES, NW = C::NW, XI = C::XI, WI = C::WI, IW = C::IW, NLI = (XI + WI) * IW;
+  constexpr int S = C::STAGES, NW = C::NW, XIW = C::XIW, WIW = C::WIW, IW = C::IW, NLI = XIW + WIW;
   constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
   // one fragment buffer for fp8 (8-register fragments) and for the 256-row tile on 16x16 MFMAs (twelve fragments
   // per K-step next to 128 accumulators), two otherwise
@@ -239,10 +239,12 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     tile_coords(a, expert_off, lin_, pt_, pf_, ex_);                                           \
   }
   // rows of the load slots this wavefront issues: load index ih -> tile row
-#define FR_SLOT_ROW(ih_, rr_, c_)                                                  \
+  // (ROWS_: rows of the tile.  With an odd number of loads per issuing wavefront the last index lies beyond the tile
+  // for the wavefronts that issue nothing; they only share the address code, and their row is clamped into the tile)
+#define FR_SLOT_ROW(ih_, rr_, c_, ROWS_)                                           \
   const int vw_ = (wave_u + ((ih_) % IW) * (NW / IW)) % NW;                        \
   const int slot_ = (((ih_) / IW) * NW + vw_) * kWave + lane;                      \
-  const int rr_ = slot_ / CPR, c_ = swizzle<CPR>(rr_, slot_ % CPR);
+  const int rr_ = min(slot_ / CPR, (ROWS_) - 1), c_ = swizzle<CPR>(rr_, slot_ % CPR);
   auto w_src_row = [&](int pf, int rr) -> int {
     if constexpr (EPI == EPI_SILU) {
       const int half = rr / (BF / 2), f = pf * (BF / 2) + rr % (BF / 2);
@@ -270,8 +272,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   // ---- address sets: A = tile being multiplied, B = the workgroup's next tile --------
   int pid_t, pid_f, expert, kb, kn, tu;  // current unit: tile, first K tile and K tile count, slice buffer
   int n_pid_t = 0, n_pid_f = 0, n_expert = 0, n_kb = 0, n_kn = 0, n_tu = -1;
-  int n_sid[XI * IW];  // sorted ids of the next tile's load rows, fetched a tile ahead
-  unsigned xsrcA[XI * IW], wsrcA[WI * IW], xsrcB[XI * IW], wsrcB[WI * IW];
+  int n_sid[XIW];  // sorted ids of the next tile's load rows, fetched a tile ahead
+  unsigned xsrcA[XIW], wsrcA[WIW], xsrcB[XIW], wsrcB[WIW];
   __amdgpu_buffer_rsrc_t xrsA, wrsA, xrsB, wrsB;
 #define FR_MAKE_SET(pt_, pf_, ex_, kb_, SIDOF, xsrc_, wsrc_, xrs_, wrs_)                                     \
   {                                                                                                          \
@@ -279,16 +281,16 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     const int64_t kfirst_ = k0 + static_cast<int64_t>(kb_) * BK;                                             \
     xrs_ = uniform_rsrc(X + xrow0_ * a.ldx, a.x_span ? a.x_span : 0xFFFFFFFFu);                              \
     wrs_ = uniform_rsrc(static_cast<const T*>(a.W) + static_cast<int64_t>(ex_) * a.w_expert_stride);         \
-    _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) {                                                 \
-      FR_SLOT_ROW(ih, rr, c)                                                                                 \
+    _Pragma("unroll") for (int ih = 0; ih < XIW; ++ih) {                                                 \
+      FR_SLOT_ROW(ih, rr, c, BT)                                                                              \
       int64_t row_ = rr;                                                                                     \
       const int sid_ = SIDOF;                                                                                \
       if (a.top_k > 0) row_ = sid_ < a.num_valid ? sid_ / a.top_k : 0;                                       \
       xsrc_[ih] = static_cast<unsigned>((row_ * a.ldx + kfirst_ + c * EPC) * static_cast<int64_t>(sizeof(T))); \
       if (a.x_span && sid_ >= a.num_valid) xsrc_[ih] = kSkipOffset;                                          \
     }                                                                                                        \
-    _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) {                                                 \
-      FR_SLOT_ROW(ih, rr, c)                                                                                 \
+    _Pragma("unroll") for (int ih = 0; ih < WIW; ++ih) {                                                 \
+      FR_SLOT_ROW(ih, rr, c, BF)                                                                              \
       wsrc_[ih] = static_cast<unsigned>(w_byte_offset(a.w_tiled, a.ldw, a.K, w_src_row(pf_, rr),             \
                                                       (kfirst_ + c * EPC) * static_cast<int64_t>(sizeof(T)), sizeof(T))); \
     }                                                                                                        \
@@ -315,14 +317,14 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
 #define FR_ISSUE_REAL(SET, tile_, slot_, q_)                                                                \
   {                                                                                                         \
     const int vwi_ = wave_u + ((q_) % IW) * (NW / IW);                                                      \
-    if ((q_) < WI * IW) {                                                                                   \
+    if ((q_) < WIW) {                                                                                   \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
           wrs##SET, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vwi_) * (kWave * 16)), \
-          16, wsrc##SET[(q_) < WI * IW ? (q_) : 0], FR_KOFF_W(tile_), 0, 0);                                      \
+          16, wsrc##SET[(q_) < WIW ? (q_) : 0], FR_KOFF_W(tile_), 0, 0);                                      \
     } else {                                                                                                \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
-          xrs##SET, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WI * IW) / IW) * NW + vwi_) * (kWave * 16)), \
-          16, xsrc##SET[(q_) < WI * IW ? 0 : (q_) - WI * IW], FR_KOFF(tile_), 0, 0);                            \
+          xrs##SET, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WIW) / IW) * NW + vwi_) * (kWave * 16)), \
+          16, xsrc##SET[(q_) < WIW ? 0 : (q_) - WIW], FR_KOFF(tile_), 0, 0);                            \
     }                                                                                                       \
   }
 #ifdef FR_ABL_NOLOAD
@@ -454,8 +456,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     }                                                                                                      \
     if (NEXT) {                                                                                            \
       FR_UNIT(unit + 1, n_pid_t, n_pid_f, n_expert, n_kb, n_kn, n_tu)                                      \
-      _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) {                                             \
-        FR_SLOT_ROW(ih, rr, c)                                                                             \
+      _Pragma("unroll") for (int ih = 0; ih < XIW; ++ih) {                                             \
+        FR_SLOT_ROW(ih, rr, c, BT)                                                                          \
         (void)c;                                                                                           \
         n_sid[ih] = a.sorted[n_pid_t * BT + rr];                                                           \
       }                                                                                                    \
@@ -499,8 +501,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
       FR_TILE(ISS_, true)                                                                                  \
       pid_t = n_pid_t; pid_f = n_pid_f; expert = n_expert; xrsA = xrsB; wrsA = wrsB;                       \
       kb = n_kb; kn = n_kn; tu = n_tu;                                                                     \
-      _Pragma("unroll") for (int ih = 0; ih < XI * IW; ++ih) xsrcA[ih] = xsrcB[ih];                        \
-      _Pragma("unroll") for (int ih = 0; ih < WI * IW; ++ih) wsrcA[ih] = wsrcB[ih];                        \
+      _Pragma("unroll") for (int ih = 0; ih < XIW; ++ih) xsrcA[ih] = xsrcB[ih];                        \
+      _Pragma("unroll") for (int ih = 0; ih < WIW; ++ih) wsrcA[ih] = wsrcB[ih];                        \
     }                                                                                                      \
     FR_TILE(ISS_, false)                                                                                   \
     FR_STAMP(2)                                                                                            \

@@ -29,6 +29,12 @@ template <typename T> struct Tiles {  // bf16 / fp16
   typedef T256 T256G;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<128, 256, 128, 2, 4, 16, 1, 3, 0, 2> T128P;  // persistent form; one wavefront per SIMD issues the loads (2-4 % over each its own); 16x16x32 MFMAs: 2-3 % over 32x32x16
+  // 160 token rows on the same three-slot ring: 159744 bytes, with the walk table all 160 KB of a CU.  A quarter more
+  // rows per pass of an expert's weight tiles through LDS, and room for the spread of the experts' loads around a
+  // multiple of 128 (n pairs on E experts: n/E +- sqrt(n/E) rows each, so with n/E = 128, 256, 512 every other expert
+  // needs one 128-row block more than n/E / 128).  Five token tiles x four weight tiles per wavefront, five of the
+  // thirteen loads per issuing wavefront and K tile for the token rows.
+  typedef Cfg<160, 256, 128, 2, 4, 16, 1, 3, 0, 2> T160P;
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 3, 3> T64;    // 3-slot ring like the 128-row tile (5 % over the register-staged form)
   typedef Cfg<64, 128, 256, 2, 2, 32, 1, 3> T64U;      // gate/up: 256-byte row segments, 4 wavefronts (another 5 %)
   typedef Cfg<32, 128, 128, 1, 4, 16, 2, 3> T32;
@@ -45,6 +51,7 @@ template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per
   typedef T256 T256S;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;
+  typedef T128P T160P;  // placeholder: 160-row blocks are for 2-byte operands (80 rows per wavefront are no multiple of the 32-row fp8 MFMA tile)
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 3, 3> T64;
   typedef Cfg<64, 128, 256, 2, 2, 32, 1, 3> T64U;
   typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;
@@ -55,7 +62,7 @@ template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per
 
 constexpr int kSmallMfmaMinK = 4096;  // K from which the 256-row tile of 2-byte operands takes the 16x16x32 MFMA form
 
-inline bool valid_block(int block) { return block == 16 || block == 32 || block == 64 || block == 128 || block == 256; }
+inline bool valid_block(int block) { return block == 16 || block == 32 || block == 64 || block == 128 || block == 160 || block == 256; }
 inline int elem_bytes(int dtype) { return dtype == FR_FP8_E4M3 ? 1 : 2; }
 inline int tile_k_bytes(int block, int dtype) { return (block == 16 || (block == 32 && dtype == FR_FP8_E4M3)) ? 256 : 128; }
 inline int k_multiple(int dtype, int block) { return tile_k_bytes(block, dtype) / elem_bytes(dtype); }
@@ -98,6 +105,13 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
         return launch_gemm_persistent<T, typename TL::T128P, EPI>(a, splits, st);
       }
       return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
+    case 160:
+      if constexpr (sizeof(T) == 2) {
+        fill(160, TL::T160P::BF, TL::T160P::BKB);
+        return launch_gemm_persistent<T, typename TL::T160P, EPI>(a, splits, st);
+      } else {
+        return fail(FR_E_SHAPE, "routing block 160 is for 2-byte operands");
+      }
     case 64:
       if (EPI == EPI_SILU && a.K % (TL::T64U::BKB / static_cast<int>(sizeof(T))) == 0) {
         fill(64, TL::T64U::BF, TL::T64U::BKB);
@@ -119,7 +133,7 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       }
       fill(16, TL::T16::BF, TL::T16::BKB);
       return launch_gemm<T, typename TL::T16, EPI>(a, splits, st);
-    default: return fail(FR_E_SHAPE, "routing block %d not in {16, 32, 64, 128, 256}", block);
+    default: return fail(FR_E_SHAPE, "routing block %d not in {16, 32, 64, 128, 160, 256}", block);
   }
 }
 
@@ -135,6 +149,9 @@ int prepare_tiles() {
     if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T256S, EPI>(a, 1, nullptr);
   }
   if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T128P, EPI>(a, 1, nullptr);
+  if constexpr (sizeof(T) == 2) {
+    if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T160P, EPI>(a, 1, nullptr);
+  }
   if (rc == FR_OK) rc = launch_gemm<T, typename TL::T128, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm<T, typename TL::T64, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm<T, typename TL::T32, EPI>(a, 1, nullptr);

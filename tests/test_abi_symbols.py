@@ -42,7 +42,7 @@ def test_host_only_calls_need_no_gpu():
     assert lib.fr_moe_align_workspace_bytes(10, 5000) == -1
     p = _native.FrMoePlan()
     assert lib.fr_moe_get_plan(64, 4096, 14336, 8, 2, _native.FR_BF16, p) == 0
-    assert p.block in (16, 32, 64, 128, 256) and p.split_k >= 1
+    assert p.block in (16, 32, 64, 128, 160, 256) and p.split_k >= 1
     assert p.sorted_len == 128 + 8 * (p.block - 1) and p.workspace_bytes > 0
     # argument errors come back as codes + message, never as aborts
     assert lib.fr_moe_get_plan(64, 4095, 14336, 8, 2, _native.FR_BF16, p) == -2
@@ -56,8 +56,10 @@ def test_host_only_calls_need_no_gpu():
 def test_plan_table():
     """The tile plan is host logic: routing block and K slices of the down projection per token count,
     as documented (Mixtral shape: 16-row blocks up to 8 pairs per expert, 32 below 26, 64 below 52 at
-    H >= 4096, 128 below 560, 256 above; the fine-grained shape with H = 2048 has no 64-row range and
-    keeps 128 rows up to 4096 pairs per expert)."""
+    H >= 4096, then 128 or - where the spread of the experts' loads around a multiple of 128 would cost
+    every other expert one block more - 160, 256 from 1200 pairs per expert on; fp8 has no 160-row tile and
+    switches from 128 to 256 at 560; the fine-grained shape with H = 2048 has no 64-row range and never
+    takes 256 rows below 4096 pairs per expert)."""
     from fast_route_amd import _native
     lib = _native.lib()
 
@@ -68,13 +70,14 @@ def test_plan_table():
         return p.block, p.split_k
 
     mix = lambda M, dt=_native.FR_BF16: plan(M, 4096, 14336, 8, 2, dt)
-    assert [mix(M)[0] for M in (1, 32, 33, 103, 104, 207, 208, 2239, 2240)] == [16, 16, 32, 32, 64, 64, 128, 128, 256]
+    assert [mix(M)[0] for M in (1, 32, 33, 103, 104, 207, 208, 460, 461, 684, 685, 768, 1024, 4096, 4799, 4800)] == \
+        [16, 16, 32, 32, 64, 64, 128, 128, 160, 160, 128, 128, 160, 160, 160, 256]
     assert mix(1) == (16, 4) and mix(2) == (16, 2) and mix(3) == (16, 4) and mix(4) == (16, 4) and mix(16) == (16, 1)
     assert mix(128) == (64, 2)
-    assert mix(4096)[1] == 1 and plan(4096, 4096, 14336, 8, 2)[0] == 256
-    assert [mix(M, _native.FR_FP8_E4M3)[0] for M in (103, 104, 207, 208)] == [32, 64, 64, 128]
+    assert mix(4096)[1] == 1 and plan(16384, 4096, 14336, 8, 2)[0] == 256
+    assert [mix(M, _native.FR_FP8_E4M3)[0] for M in (103, 104, 207, 208, 512, 2239, 2240)] == [32, 64, 64, 128, 128, 128, 256]
     fine = lambda M: plan(M, 2048, 1408, 64, 6)[0]
-    assert [fine(M) for M in (85, 86, 341, 342, 43690, 43691)] == [16, 32, 32, 128, 128, 256]
+    assert [fine(M) for M in (85, 86, 341, 342, 1220, 1221, 43690, 43691)] == [16, 32, 32, 128, 128, 160, 160, 256]
     # the scratch for splitting the last round exists exactly for 128- and 256-row blocks with a long K
     p = _native.FrMoePlan()
     lib.fr_moe_get_plan(4096, 4096, 14336, 8, 2, _native.FR_BF16, p)
@@ -119,7 +122,8 @@ def test_bench_refuses_more_than_one_gpu():
 
 def test_recorded_traffic_matches_profiles_file():
     """bench.py reports roofline.traffic from profiles/hbm_traffic.json for the workloads recorded there,
-    as long as the kernel sources are the ones the record was measured with."""
+    as long as the grouped-GEMM kernel sources are the ones the record was measured with and the plan still
+    picks the routing block (the tile) that was measured."""
     import importlib.util
     import json
     import os
@@ -131,9 +135,11 @@ def test_recorded_traffic_matches_profiles_file():
     key = "moe_layer_tflops_mixtral_bf16_M4096"
     assert rec[key]["traffic_bytes"] == rec[key]["fetch_bytes"] + rec[key]["write_bytes"]
     # the record counts only for the kernel sources it was measured with
+    block = rec[key]["block"]
     want = rec[key]["traffic_bytes"] if rec.get("kernel_sources_sha") == mod.kernel_sources_sha() else None
-    assert mod.recorded_traffic(key) == want
-    assert mod.recorded_traffic("no_such_workload") is None
+    assert mod.recorded_traffic(key, block) == want
+    assert mod.recorded_traffic(key, block + 1) is None
+    assert mod.recorded_traffic("no_such_workload", block) is None
 
 
 def test_tunables_override_the_plan_and_reset():
@@ -149,14 +155,14 @@ def test_tunables_override_the_plan_and_reset():
         return p
 
     base = plan(4096)
-    assert (base.block, base.split_k) == (256, 1) and base.tail_bytes > 0
+    assert (base.block, base.split_k) == (160, 1) and base.tail_bytes > 0
     try:
         fr.set_tunables(block=128, split_k=3)
         p = plan(4096)
         assert (p.block, p.split_k) == (128, 3) and p.sorted_len == 8192 + 8 * 127
         assert fr.get_tunables() == {"block": 128, "split_k": 3, "group_m": 0, "no_tail_split": False, "epilogue_combine": False}
         with fr.tunables(no_tail_split=True):
-            assert plan(4096).tail_bytes == 0 and plan(4096).block == 256  # the context replaces, then restores
+            assert plan(4096).tail_bytes == 0 and plan(4096).block == 160  # the context replaces, then restores
         assert plan(4096).block == 128
         fr.set_tunables(split_k=64)  # as many slices as keep 8 K tiles each: 14336 / (8 * 64) = 28
         assert plan(4096).split_k == 28

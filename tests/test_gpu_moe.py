@@ -166,7 +166,7 @@ def test_layer_with_64_row_blocks(native, dtype):
     _assert_close(out, oracle.fused_moe(x, w1, w2, logits, k, True), dtype, "64-row blocks")
 
 
-@pytest.mark.parametrize("block", [16, 32, 64, 128, 256])
+@pytest.mark.parametrize("block", [16, 32, 64, 128, 160, 256])
 def test_op_level_chain_matches_reference_layer_recipe(native, block):
     """The reference layer spelled with its own ops (layers/stable_route.py:82-102):
     align -> grouped GEMM -> silu_and_mul -> grouped GEMM * weight -> sum."""
@@ -220,11 +220,12 @@ def test_block_256_several_tiles_per_workgroup(native, dtype):
     _assert_close(out, oracle.fused_moe(x, w1, w2, logits, k, True), dtype, "layer")
 
 
+@pytest.mark.parametrize("rows", [256, 160])
 @pytest.mark.parametrize("case", ["gate_up_after_whole_tile", "down_first_unit", "with_and_without_scratch"])
-def test_last_round_of_tiles_split_along_k(native, rows256, case):
-    """256-row tiles that only partly fill the last round of workgroups are cut along K over
+def test_last_round_of_tiles_split_along_k(native, rows, case):
+    """256-row (and 160-row) tiles that only partly fill the last round of workgroups are cut along K over
     the idle ones and summed by a second launch.  Routing is constructed so that the tile
-    counts are exact (k = 1, every expert a whole number of 256-token blocks):
+    counts are exact (k = 1, every expert a whole number of `rows`-token blocks):
     gate_up_after_whole_tile - 17 blocks x 16 feature tiles = 272 tiles, 34 per XCD: one whole
       round of 32 and 2 tiles cut into 8 K slices each (K = 4096 is 64 K tiles);
     down_first_unit - 8 blocks x 2 feature tiles over F = 4096: 2 tiles per XCD in 8 slices
@@ -233,31 +234,34 @@ def test_last_round_of_tiles_split_along_k(native, rows256, case):
       to fp32 summation order (same bf16 result up to one rounding)."""
     from fast_route_amd import _native as N, fused_experts
     from fast_route_amd.layers.fused_moe import plan
-    _say("tail split " + case)
+    import fast_route_amd as fr
+    _say(f"tail split {case} rows={rows}")
     dtype = torch.bfloat16
     if case == "down_first_unit":
         H, Fd, E, blocks = 512, 4096, 2, (5, 3)
     else:
         H, Fd, E, blocks = 4096, 2048, 3, (9, 0, 8)
-    M = 256 * sum(blocks)
+    M = rows * sum(blocks)
     g = torch.Generator().manual_seed(77)
     x = torch.randn(M, H, generator=g).to(dtype)
     w1 = (torch.randn(E, 2 * Fd, H, generator=g) * 0.02).to(dtype)
     w2 = (torch.randn(E, H, Fd, generator=g) * 0.02).to(dtype)
-    ids = torch.cat([torch.full((256 * b,), e, dtype=torch.int32) for e, b in enumerate(blocks)])
+    ids = torch.cat([torch.full((rows * b,), e, dtype=torch.int32) for e, b in enumerate(blocks)])
     ids = ids[torch.randperm(M, generator=g)].view(M, 1)
     w = (torch.rand(M, 1, generator=g) + 0.5).float()
-    p = plan(M, H, Fd, E, 1, dtype)
-    assert p.block == 256 and p.tail_bytes > 0 and p.split_k == 1
+    with fr.tunables(block=rows):  # the plan itself keeps a short gate/up K on smaller blocks
+        p = plan(M, H, Fd, E, 1, dtype)
+    assert p.block == rows and p.tail_bytes > 0 and p.split_k == 1
     xd, w1d, w2d, wd, idd = x.cuda(), w1.cuda(), w2.cuda(), w.cuda(), ids.cuda()
     if case != "with_and_without_scratch":
-        out = fused_experts(xd, w1d, w2d, wd, idd)
+        with fr.tunables(block=rows):
+            out = fused_experts(xd, w1d, w2d, wd, idd)
         torch.cuda.synchronize()
         _assert_close(out, oracle.moe_experts(x, w1, w2, w, ids), dtype, case)
         return
     from fast_route_amd.ops.fused_moe import moe_align_block_size
     lib, st = N.lib(), torch.cuda.current_stream().cuda_stream
-    s, e, npost = moe_align_block_size(idd, 256, E)
+    s, e, npost = moe_align_block_size(idd, rows, E)
     tail = torch.empty(p.tail_bytes, dtype=torch.uint8, device="cuda")
     res = []
     for tptr in (None, tail.data_ptr()):
@@ -265,9 +269,9 @@ def test_last_round_of_tiles_split_along_k(native, rows256, case):
         partial = torch.empty(M * H, dtype=torch.float32, device="cuda")
         out = torch.empty(M, H, dtype=dtype, device="cuda")
         N.check(lib.fr_moe_gateup_silu(xd.data_ptr(), w1d.data_ptr(), s.data_ptr(), e.data_ptr(), npost.data_ptr(), M, H,
-                                       Fd, E, 1, 256, N.FR_BF16, act.data_ptr(), tptr, st))
+                                       Fd, E, 1, rows, N.FR_BF16, act.data_ptr(), tptr, st))
         N.check(lib.fr_moe_down_combine(act.data_ptr(), w2d.data_ptr(), wd.data_ptr(), s.data_ptr(), e.data_ptr(),
-                                        npost.data_ptr(), M, H, Fd, E, 1, 256, 1, N.FR_BF16, partial.data_ptr(),
+                                        npost.data_ptr(), M, H, Fd, E, 1, rows, 1, N.FR_BF16, partial.data_ptr(),
                                         out.data_ptr(), tptr, st))
         torch.cuda.synchronize()
         res.append((act.float().cpu(), out.float().cpu()))
@@ -383,7 +387,7 @@ def test_layer_under_graph_capture(native, M):
     _assert_close(out, oracle.fused_moe(xd.cpu(), w1, w2, ld.cpu(), k, True), dtype, "graph replay")
 
 
-@pytest.mark.parametrize("block", [128, 256])
+@pytest.mark.parametrize("block", [128, 160, 256])
 def test_grouped_gemm_with_blocks_in_any_order(native, block):
     """The op-level GEMM only needs every block to belong to one expert; routing arrays whose
     blocks are not in ascending expert order (here: reversed) are legal input.  The persistent
@@ -600,7 +604,8 @@ def test_tunables_and_prepare(native):
     _assert_close(base, ref, dtype, "library plan")
     try:
         for kw in ({"block": 16}, {"block": 32, "split_k": 3}, {"block": 64, "group_m": 1}, {"block": 128, "split_k": 2},
-                   {"block": 256, "no_tail_split": True}, {"block": 256, "group_m": 3}, {"split_k": 4}, {"group_m": 64}):
+                   {"block": 256, "no_tail_split": True}, {"block": 256, "group_m": 3}, {"split_k": 4}, {"group_m": 64},
+                   {"block": 160}, {"block": 160, "split_k": 2}):
             _say(f"tunables {kw}")
             with fr.tunables(**kw):
                 out = fused_moe(xd, w1d, w2d, ld, 2, True)
@@ -612,10 +617,9 @@ def test_tunables_and_prepare(native):
     assert torch.equal(fused_moe(xd, w1d, w2d, ld, 2, True), base)
 
 
-@pytest.mark.parametrize("block", [128, 256])
-@pytest.mark.parametrize("kind", ["bf16", "fp8"])
+@pytest.mark.parametrize("block,kind", [(128, "bf16"), (160, "bf16"), (256, "bf16"), (128, "fp8"), (256, "fp8")])
 def test_persistent_tiles_alternating_half_empty_and_full_blocks(native, block, kind):
-    """The persistent 128- and 256-row kernels let the wavefronts of a block's upper half skip their fragment
+    """The persistent 128-, 160- and 256-row kernels let the wavefronts of a block's upper half skip their fragment
     reads and MFMAs when that half holds only padding, and pick the fragments up again when their next block
     has rows.  64 experts with one routing block each, a seeded mix of full blocks and blocks filled to less
     than half, 8 feature tiles per block: every workgroup walks several units and meets both transitions."""
