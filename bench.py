@@ -263,11 +263,11 @@ def kernel_roofline(shape, rec, fp8=False):
     byts = rec["active_experts"] * 2 * F * H * eb + M * H * eb + M * topk * F * 2
     peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
     # which kernel the library picks for the gate/up GEMM: weight rows against token rows for up to 4
-    # tokens of 2-byte operands with H = 4096, 5120, 6144, 7168 or 8192, the persistent tile kernel for 128-row blocks
-    # and for 256-row blocks of 2-byte operands, the plain tile kernel otherwise
+    # tokens of 2-byte operands with H = 4096, 5120, 6144, 7168 or 8192, the persistent tile kernel for 128- and 160-row
+    # blocks and for 256-row blocks of 2-byte operands, the plain tile kernel otherwise
     if not fp8 and M <= 4 and H >= 4096 and H % 512 == 0 and any(H // 512 % c == 0 for c in (5, 6, 7, 8)) and M * H * 2 <= 65536:
         name = "gateup_rows_kernel"
-    elif rec["block"] == 128 or (rec["block"] == 256 and not fp8):
+    elif rec["block"] in (128, 160) or (rec["block"] == 256 and not fp8):
         name = "moe_gemm_persistent_kernel<EPI_SILU>"
     else:
         name = "moe_gemm_kernel<EPI_SILU>"

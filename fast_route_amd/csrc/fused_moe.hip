@@ -122,7 +122,7 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   else if (avg < 52 && H >= 4096) block = 64;
   else if (avg < t256) block = 128;
   else block = 256;
-  // 160-row blocks (2-byte operands, a gate/up K of at least 32 K tiles): the same three-slot ring as the 128-row
+  // 160-row blocks (a gate/up K of at least 32 K tiles): the same three-slot ring as the 128-row
   // tile with a quarter more rows per pass of an expert's weights through LDS.  Under uniform routing an expert
   // gets avg +- sqrt(avg) pairs, so with avg = 128, 256, 384, 512 every other expert needs one 128-row block more
   // than avg / 128; 160 rows absorb the spread.  Taken where the expected number of blocks per expert drops by a
@@ -136,8 +136,12 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // With a 160-row candidate the 256-row tile takes over at 1200 pairs per expert (H >= 4096).  Below 112 pairs per expert one
   // block holds an expert either way and the smaller tile is cheaper (256 / 384 tokens: 548 / 556, 580 / 602 us);
   // with H = 1024 (16 K tiles) the 160-row tile loses (700 tokens: 85 / 96 us).
-  if ((block == 128 || block == 256) && (dtype == FR_BF16 || dtype == FR_F16) && H >= 2048 && E <= 1022 && avg >= 112 &&
-      avg < (H >= 4096 ? 1200.0 : t256)) {
+  // fp8 (16x16x128 MFMAs for this tile; its gate/up kernel spills 46 registers): only where a fifth of the blocks
+  // go - 512 / 1024 tokens 435 / 392 and 543 / 505 us, but 2048 tokens 853 / 877 - and never instead of 256 rows
+  // (4096 tokens: 1506 against 1495 us).
+  const bool two_byte = dtype == FR_BF16 || dtype == FR_F16;
+  if ((block == 128 || (block == 256 && two_byte)) && H >= 2048 && F >= 1024 && E <= 1022 && avg >= 112 &&
+      avg < (two_byte && H >= 4096 ? 1200.0 : t256)) {
     const double sigma = sqrt(avg * (1.0 - 1.0 / E)) + 1e-9;
     auto tail = [&](double x) { return 0.5 * erfc((x - avg) / (sigma * 1.4142135623730951)); };  // P(pairs of an expert > x)
     auto expected = [&](int rows) {  // expected multiples of `rows` that hold an expert's pairs
@@ -147,10 +151,12 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
     };
     const double b128 = expected(128), b160 = expected(160);
     const double c128 = expected(64) * 64, c160 = expected(80) * 80;
-    const bool take160 = b160 * 1.1 < b128 || c160 <= 0.98 * c128;
+    const bool take160 = two_byte ? (b160 * 1.1 < b128 || c160 <= 0.98 * c128) : b160 * 1.2 < b128;
     if (take160) block = 160;
   }
   if (g_tunables.block) block = g_tunables.block;
+  // the fp8 160-row tile exists in the persistent form only (five K tiles per K slice at least, 1022 experts at most)
+  if (block == 160 && !two_byte && (H < 640 || F < 1024 || E > 1022)) block = 128;
   // Down projection: N = H gives few feature tiles, so K is split.
   const int bf = block == 16 ? 64 : (block == 32 ? 128 : 256);
   const int64_t blocks = n <= E ? n : (block >= 128 ? ceil_div(n, block) + E / 2 : E);

@@ -119,7 +119,7 @@ int64_t tail_scratch_bytes(int block, int dtype, int64_t K, int64_t N, bool gate
   static_assert(Tiles<fp8_t>::T256::BF == C::BF && Tiles<fp8_t>::T256::BKB == C::BKB, "same K tile and feature tile");
   const bool two_byte = dtype == FR_BF16 || dtype == FR_F16;
   if (!two_byte && dtype != FR_FP8_E4M3) return 0;
-  if (!((block == 256 && (two_byte || !gateup)) || block == 128 || (block == 160 && two_byte))) return 0;
+  if (!((block == 256 && (two_byte || !gateup)) || block == 128 || block == 160)) return 0;
   const int64_t bk = C::BKB / elem_bytes(dtype), cols = gateup ? C::BF / 2 : C::BF;
   if (K / bk < kTailMinTiles || N % cols != 0) return 0;
   return static_cast<int64_t>(kTailUnits) * C::BT * C::BF * 4;  // sized for the larger tile

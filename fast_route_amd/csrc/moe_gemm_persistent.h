@@ -664,14 +664,26 @@ int launch_gemm_persistent(const GemmArgs& a_in, int splits, hipStream_t st) {
   GemmArgs a = a_in;
   constexpr int BK = C::BKB / static_cast<int>(sizeof(T));
   const int last_k = a.K - (splits - 1) * a.k_per_split;  // K range of the last split
+  // The plain kernel double-buffers its fragments over an even number of K-steps per K tile; a tile without that
+  // (fp8 on the 16x16x128 MFMA: one K-step per 128-byte K tile) exists in the persistent form only.
+  constexpr bool kPlainForm = (C::CPR / (C::KGROUPS * Elem<T>::FC)) % 2 == 0;
+  auto plain = [&](const GemmArgs& g) -> int {
+    if constexpr (kPlainForm) {
+      return launch_gemm<T, C, EPI>(g, splits, st);
+    } else {
+      if (g.setup_only) return FR_OK;
+      return fail(FR_E_SHAPE, "the %d-row tile of this element type needs at least %d K tiles per K slice and at most %d experts",
+                  C::BT, C::STAGES + 2, kMaxExperts);
+    }
+  };
   if (a.setup_only) {  // both forms a launch may take
     int resident = 0;
     const int rc = persistent_grid<T, C, EPI>(&resident);
-    return rc != FR_OK ? rc : launch_gemm<T, C, EPI>(a, splits, st);
+    return rc != FR_OK ? rc : plain(a);
   }
   if (a.k_per_split / BK < C::STAGES + 2 || last_k / BK < C::STAGES + 2 || a.num_experts < 1 || a.num_experts > kMaxExperts) {
     a.tail_ws = nullptr;
-    return launch_gemm<T, C, EPI>(a, splits, st);
+    return plain(a);
   }
   const int64_t x_rows = a.top_k > 0 ? a.num_valid / a.top_k : C::BT;
   const int64_t w_rows = EPI == EPI_SILU ? 2 * static_cast<int64_t>(a.N) : a.N;

@@ -51,7 +51,7 @@ template <> struct Tiles<fp8_t> {  // the 16x16x128 MFMA eats 256 bytes of K per
   typedef T256 T256S;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 3> T128;
   typedef Cfg<128, 256, 128, 2, 4, 32, 1, 3, 0, 2> T128P;
-  typedef T128P T160P;  // placeholder: 160-row blocks are for 2-byte operands (80 rows per wavefront are no multiple of the 32-row fp8 MFMA tile)
+  typedef Cfg<160, 256, 128, 2, 4, 16, 1, 3, 0, 2> T160P;  // on the 16x16x128 MFMA (80 rows per wavefront are no multiple of 32)
   typedef Cfg<64, 256, 128, 2, 4, 32, 1, 3, 3> T64;
   typedef Cfg<64, 128, 256, 2, 2, 32, 1, 3> T64U;
   typedef Cfg<32, 128, 256, 1, 4, 16, 2, 2> T32;
@@ -106,12 +106,8 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       }
       return launch_gemm<T, typename TL::T128, EPI>(a, splits, st);
     case 160:
-      if constexpr (sizeof(T) == 2) {
-        fill(160, TL::T160P::BF, TL::T160P::BKB);
-        return launch_gemm_persistent<T, typename TL::T160P, EPI>(a, splits, st);
-      } else {
-        return fail(FR_E_SHAPE, "routing block 160 is for 2-byte operands");
-      }
+      fill(160, TL::T160P::BF, TL::T160P::BKB);
+      return launch_gemm_persistent<T, typename TL::T160P, EPI>(a, splits, st);
     case 64:
       if (EPI == EPI_SILU && a.K % (TL::T64U::BKB / static_cast<int>(sizeof(T))) == 0) {
         fill(64, TL::T64U::BF, TL::T64U::BKB);
@@ -149,9 +145,7 @@ int prepare_tiles() {
     if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T256S, EPI>(a, 1, nullptr);
   }
   if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T128P, EPI>(a, 1, nullptr);
-  if constexpr (sizeof(T) == 2) {
-    if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T160P, EPI>(a, 1, nullptr);
-  }
+  if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T160P, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm<T, typename TL::T128, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm<T, typename TL::T64, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm<T, typename TL::T32, EPI>(a, 1, nullptr);

@@ -15,7 +15,7 @@ from . import _native as N
 def set_tunables(block: int = 0, split_k: int = 0, group_m: int = 0, no_tail_split: bool = False,
                  epilogue_combine: bool = False) -> None:
     """0 leaves a choice to the library.  block: routing block / token rows per tile
-    (16, 32, 64, 128, 256); split_k: K slices of the down projection; group_m: token blocks
+    (16, 32, 64, 128, 160, 256); split_k: K slices of the down projection; group_m: token blocks
     walked together over the feature tiles; no_tail_split: never split the last round of tiles;
     epilogue_combine: top-2 combine by atomic adds in the down GEMM's epilogue (measured slower than the combine kernel)."""
     t = N.FrMoeTunables(int(block), int(split_k), int(group_m), int(bool(no_tail_split)), int(bool(epilogue_combine)))

@@ -91,7 +91,8 @@ int fr_moe_align(const void* topk_ids, int ids_dtype, int64_t n, int E, int bloc
  *   A [*, K] (row stride lda), B [E, N, K] dense, C [num_valid, N] dense.
  * Replaces: invoke_fused_moe_kernel / fused_moe_kernel,
  * fast_route/fast_route/ops/fused_moe.py:178-214 and :10-130.
- * Limits: K % 64 == 0 (K % 128 == 0 for block 16), N % 4 == 0, block in {16, 32, 64, 128, 256};
+ * Limits: K % 64 == 0 (K % 128 == 0 for block 16), N % 4 == 0, block in {16, 32, 64, 128, 160, 256} (fp8 with block 160:
+ * K >= 640 and E <= 1022);
  * dtype in {FR_F16, FR_BF16}. */
 int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, void* C,
                         const float* topk_weights, const int32_t* sorted_token_ids,
@@ -155,7 +156,7 @@ int fr_moe_prepare(int dtype);
 /* Study knobs of the tile plan, process-wide (set them from one thread while no call is in
  * flight; they are read when a call is made, not when its kernels run).  0 in a field leaves
  * that choice to the library.
- *   block      routing block = token rows per GEMM tile: 16, 32, 64, 128 or 256
+ *   block      routing block = token rows per GEMM tile: 16, 32, 64, 128, 160 or 256
  *   split_k    K slices of the down projection, 1..64 (1 also switches the last-round split on
  *              where the tile supports it, as the plan itself would)
  *   group_m    token blocks walked together over the feature tiles (L2 sharing of weight tiles),

@@ -90,7 +90,7 @@ def test_fp8_layer_with_64_row_blocks(native):
 
 
 def test_fp8_mixtral_shape_sampled(native):
-    """Full fp8 workload shape (H4096 F14336 E8 top2), M in {16, 128, 256, 4096}: sampled tokens vs the
+    """Full fp8 workload shape (H4096 F14336 E8 top2), M in {16, 128, 256, 512, 1024, 4096} (512 and 1024: 160-row blocks): sampled tokens vs the
     oracle.  At M=4096 the down projection runs the persistent form with its last round of tiles
     split along K."""
     from fast_route_amd import fused_moe_fp8, prepare_weights_fp8
@@ -101,7 +101,7 @@ def test_fp8_mixtral_shape_sampled(native):
     w1q, w1s, w2q, w2s = prepare_weights_fp8(w1, w2)
     w1c, w2c = w1.cpu(), w2.cpu()
     wq = oracle.quantize_weights_fp8(w1c, w2c)  # once: 1.4e9 weights through the CPU encoder
-    for M in (16, 128, 256, 4096):
+    for M in (16, 128, 256, 512, 1024, 4096):
         _say(f"fp8 mixtral M={M}")
         x = torch.randn(M, H, generator=g, device="cuda").bfloat16()
         logits = torch.randn(M, E, generator=g, device="cuda")

@@ -617,7 +617,7 @@ def test_tunables_and_prepare(native):
     assert torch.equal(fused_moe(xd, w1d, w2d, ld, 2, True), base)
 
 
-@pytest.mark.parametrize("block,kind", [(128, "bf16"), (160, "bf16"), (256, "bf16"), (128, "fp8"), (256, "fp8")])
+@pytest.mark.parametrize("block,kind", [(128, "bf16"), (160, "bf16"), (256, "bf16"), (128, "fp8"), (160, "fp8"), (256, "fp8")])
 def test_persistent_tiles_alternating_half_empty_and_full_blocks(native, block, kind):
     """The persistent 128-, 160- and 256-row kernels let the wavefronts of a block's upper half skip their fragment
     reads and MFMAs when that half holds only padding, and pick the fragments up again when their next block
@@ -626,6 +626,8 @@ def test_persistent_tiles_alternating_half_empty_and_full_blocks(native, block, 
     import fast_route_amd as fr
     from fast_route_amd import fused_experts, fused_moe_fp8, prepare_weights_fp8
     E, H, Fd = 64, 512, 1024
+    if (block, kind) == (160, "fp8"):
+        H = 1024  # that tile has no plain form: five K tiles of 128 bytes per K slice at least
     rng = np.random.default_rng(block)
     counts = np.where(rng.random(E) < 0.5, block, rng.integers(1, block // 2 + 1, E))
     ids = torch.from_numpy(np.repeat(np.arange(E), counts)).int()
