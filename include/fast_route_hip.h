@@ -91,8 +91,7 @@ int fr_moe_align(const void* topk_ids, int ids_dtype, int64_t n, int E, int bloc
  *   A [*, K] (row stride lda), B [E, N, K] dense, C [num_valid, N] dense.
  * Replaces: invoke_fused_moe_kernel / fused_moe_kernel,
  * fast_route/fast_route/ops/fused_moe.py:178-214 and :10-130.
- * Limits: K % 64 == 0 (K % 128 == 0 for block 16), N % 4 == 0, block in {16, 32, 64, 128, 160, 256} (fp8 with block 160:
- * K >= 640 and E <= 1022);
+ * Limits: K % 64 == 0 (K % 128 == 0 for block 16), N % 4 == 0, block in {16, 32, 64, 128, 160, 256};
  * dtype in {FR_F16, FR_BF16}. */
 int fr_moe_grouped_gemm(const void* A, int64_t lda, const void* B, void* C,
                         const float* topk_weights, const int32_t* sorted_token_ids,
@@ -267,7 +266,9 @@ int fr_quant_e4m3_rows(const void* x, int dtype, int64_t rows, int64_t K, int64_
 /* fp8 forms of fr_moe_gateup_silu / fr_moe_down_combine: operands are e4m3
  * codes with one fp32 scale per row (x_scale[M], w1_scale[E, 2F], act_scale
  * [sorted_len], w2_scale[E, H]); act is written / read in bf16 resp. e4m3;
- * H and F must be multiples of 256.  `tail_ws` as for fr_moe_down_combine. */
+ * H and F must be multiples of 256.  `tail_ws` as for fr_moe_down_combine.
+ * block 160 (a tile without a plain form for fp8) needs K >= 640 per K slice and E <= 1022; fr_moe_get_plan
+ * never hands out a block these calls refuse. */
 int fr_moe_gateup_silu_fp8(const void* xq, const float* x_scale, const void* w1q, const float* w1_scale,
                            const int32_t* sorted_token_ids, const int32_t* expert_ids,
                            const int32_t* num_tokens_post_pad, int64_t M, int64_t H, int64_t F, int E,
