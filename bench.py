@@ -673,15 +673,21 @@ def main():
     if args.prepared and fp8 is None:
         from fast_route_amd import prepare_weights
         w1, w2, prepared = prepare_weights(w1, w2, args.prepared)
-    head, layer = measure(torch, N, shape, args.tokens, w1, w2, args.steps, args.warmup, args.seed, fp8, flush=flush, prepared=prepared)
+    # Every point - the headline included - is W warm-up passes and then K timed passes of its own.  The points are
+    # taken in the sweep's order (ascending token counts), the headline at its place among them: a process's first
+    # launches run on a device whose clocks have not settled yet (a point measured first reads 2-7 % slower than the
+    # same point measured later in the same process).  Without the sweep the headline is the only point.
+    head = layer = None
     sweep = []
     if not args.no_sweep:
         for M in sweep_ms:
-            if M == args.tokens:
-                sweep.append(head)
-                continue
-            rec, _ = measure(torch, N, shape, M, w1, w2, args.steps, args.warmup, args.seed, fp8, flush=flush, prepared=prepared)
+            rec, lay = measure(torch, N, shape, M, w1, w2, args.steps, args.warmup, args.seed, fp8, flush=flush, prepared=prepared)
             sweep.append(rec)
+            if M == args.tokens:
+                head, layer = rec, lay
+            del lay
+    if head is None:
+        head, layer = measure(torch, N, shape, args.tokens, w1, w2, args.steps, args.warmup, args.seed, fp8, flush=flush, prepared=prepared)
     result = {
         "metric": "moe_layer_tflops_%s_%s_M%d" % (args.shape, args.dtype, args.tokens),
         "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -125,8 +125,8 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // 160-row blocks (a gate/up K of at least 32 K tiles): the same three-slot ring as the 128-row
   // tile with a quarter more rows per pass of an expert's weights through LDS.  Under uniform routing an expert
   // gets avg +- sqrt(avg) pairs, so with avg = 128, 256, 384, 512 every other expert needs one 128-row block more
-  // than avg / 128; 160 rows absorb the spread.  Taken where the expected number of blocks per expert drops by a
-  // tenth or more, or the expected rows the MFMAs multiply (whole half-blocks: a wavefront row is skipped when
+  // than avg / 128; 160 rows absorb the spread.  Taken where the expected number of blocks per expert drops by an
+  // eighth or more (1 / 1.15), or the expected rows the MFMAs multiply (whole half-blocks: a wavefront row is skipped when
   // all its rows are padding) by 2 %; measured on 8 experts, H = 4096, 128 / 160 / 256 rows:
   //   tokens  512  681 / 618         us      1536  1143 / 1112 / 1132       3072        1906 / 1939
   //           640  753 / 749                 1792  1236 / 1179 / 1192       4096        2433 / 2485
@@ -151,7 +151,7 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
     };
     const double b128 = expected(128), b160 = expected(160);
     const double c128 = expected(64) * 64, c160 = expected(80) * 80;
-    const bool take160 = two_byte ? (b160 * 1.1 < b128 || c160 <= 0.98 * c128) : b160 * 1.2 < b128;
+    const bool take160 = two_byte ? (b160 * 1.15 < b128 || c160 <= 0.98 * c128) : b160 * 1.2 < b128;
     if (take160) block = 160;
   }
   if (g_tunables.block) block = g_tunables.block;

@@ -70,14 +70,14 @@ def test_plan_table():
         return p.block, p.split_k
 
     mix = lambda M, dt=_native.FR_BF16: plan(M, 4096, 14336, 8, 2, dt)
-    assert [mix(M)[0] for M in (1, 32, 33, 103, 104, 207, 208, 460, 461, 684, 685, 768, 1024, 4096, 4799, 4800)] == \
-        [16, 16, 32, 32, 64, 64, 128, 128, 160, 160, 128, 128, 160, 160, 160, 256]
+    assert [mix(M)[0] for M in (1, 32, 33, 103, 104, 207, 208, 469, 470, 670, 671, 768, 1024, 2048, 4096, 4799, 4800)] == \
+        [16, 16, 32, 32, 64, 64, 128, 128, 160, 160, 128, 128, 160, 128, 160, 160, 256]
     assert mix(1) == (16, 4) and mix(2) == (16, 2) and mix(3) == (16, 4) and mix(4) == (16, 4) and mix(16) == (16, 1)
     assert mix(128) == (64, 2)
     assert mix(4096)[1] == 1 and plan(16384, 4096, 14336, 8, 2)[0] == 256
     assert [mix(M, _native.FR_FP8_E4M3)[0] for M in (103, 104, 207, 208, 512, 768, 1024, 2048, 2240)] == [32, 64, 64, 128, 160, 128, 160, 128, 256]
     fine = lambda M: plan(M, 2048, 1408, 64, 6)[0]
-    assert [fine(M) for M in (85, 86, 341, 342, 1220, 1221, 43690, 43691)] == [16, 32, 32, 128, 128, 160, 160, 256]
+    assert [fine(M) for M in (85, 86, 341, 342, 1246, 1247, 43690, 43691)] == [16, 32, 32, 128, 128, 160, 160, 256]
     # the scratch for splitting the last round exists exactly for 128- and 256-row blocks with a long K
     p = _native.FrMoePlan()
     lib.fr_moe_get_plan(4096, 4096, 14336, 8, 2, _native.FR_BF16, p)

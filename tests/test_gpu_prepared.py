@@ -120,14 +120,14 @@ def test_fused_experts_and_inplace_with_prepared_weights(native):
 
 def test_mixtral_width_with_prepared_weights(native):
     """Full Mixtral width (H 4096, F 14336) on two experts: 512-byte K tiles of the 16- and 32-row gate/up GEMMs,
-    the 64-row tiles, the persistent 128- and 256-row tiles with their last-round split."""
+    the 64-row tiles, the persistent 128-, 160- and 256-row tiles with their last-round split."""
     from fast_route_amd import fused_moe, prepare_weights
     H, Fd, E = 4096, 14336, 2
     g = torch.Generator().manual_seed(11)
     w1 = (torch.randn(E, 2 * Fd, H, generator=g) * 0.02).to(torch.bfloat16).cuda()
     w2 = (torch.randn(E, H, Fd, generator=g) * 0.02).to(torch.bfloat16).cuda()
     w1p, w2p, flags = prepare_weights(w1, w2, "both")
-    for M in (6, 20, 40, 150, 520, 600):  # 600: 256-row blocks (16x16x32 form)
+    for M in (6, 20, 40, 150, 520, 600, 1300):  # 520 / 600: 160-row blocks; 1300: 256-row blocks (16x16x32 form)
         _say(f"prepared Mixtral width M={M}")
         x = torch.randn(M, H, generator=g).to(torch.bfloat16).cuda()
         logits = torch.randn(M, E, generator=g).cuda()
