@@ -275,12 +275,17 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   int n_sid[XIW];  // sorted ids of the next tile's load rows, fetched a tile ahead
   unsigned xsrcA[XIW], wsrcA[WIW], xsrcB[XIW], wsrcB[WIW];
   __amdgpu_buffer_rsrc_t xrsA, wrsA, xrsB, wrsB;
-#define FR_MAKE_SET(pt_, pf_, ex_, kb_, SIDOF, xsrc_, wsrc_, xrs_, wrs_)                                     \
+  // the expert of the tile has ONE token block: each of its weight tiles is read by one tile only, and marked
+  // non-temporal the stream does not displace the token rows and its own neighbours in L2
+  bool ntA = false, ntB = false;
+  constexpr bool NTW = BT < 256;  // the 256-row tiles have no register to spare for the second form of the loads
+#define FR_MAKE_SET(pt_, pf_, ex_, kb_, SIDOF, xsrc_, wsrc_, xrs_, wrs_, nt_)                                   \
   {                                                                                                          \
     const int64_t xrow0_ = a.top_k > 0 ? 0 : static_cast<int64_t>(pt_) * BT;                                 \
     const int64_t kfirst_ = k0 + static_cast<int64_t>(kb_) * BK;                                             \
     xrs_ = uniform_rsrc(X + xrow0_ * a.ldx, a.x_span ? a.x_span : 0xFFFFFFFFu);                              \
     wrs_ = uniform_rsrc(static_cast<const T*>(a.W) + static_cast<int64_t>(ex_) * a.w_expert_stride);         \
+    nt_ = NTW && !expert_off[kMaxExperts + 1] && expert_off[(ex_) + 1] - expert_off[ex_] == 1;               \
     _Pragma("unroll") for (int ih = 0; ih < XIW; ++ih) {                                                 \
       FR_SLOT_ROW(ih, rr, c, BT)                                                                              \
       int64_t row_ = rr;                                                                                     \
@@ -296,7 +301,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     }                                                                                                        \
   }
   FR_UNIT(0, pid_t, pid_f, expert, kb, kn, tu)
-  FR_MAKE_SET(pid_t, pid_f, expert, kb, a.sorted[pid_t * BT + rr], xsrcA, wsrcA, xrsA, wrsA)
+  FR_MAKE_SET(pid_t, pid_f, expert, kb, a.sorted[pid_t * BT + rr], xsrcA, wsrcA, xrsA, wrsA, ntA)
 
   // Measurement switches (compile time; results are WRONG with any of them, only timings mean something):
   //   FR_ABL_NOLOAD  the ring is filled once and never refilled: MFMAs + fragment reads + barriers on real data
@@ -318,9 +323,14 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   {                                                                                                         \
     const int vwi_ = wave_u + ((q_) % IW) * (NW / IW);                                                      \
     if ((q_) < WIW) {                                                                                   \
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
-          wrs##SET, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vwi_) * (kWave * 16)), \
-          16, wsrc##SET[(q_) < WIW ? (q_) : 0], FR_KOFF_W(tile_), 0, 0);                                      \
+      if (NTW && nt##SET)                                                                                   \
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                           \
+            wrs##SET, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vwi_) * (kWave * 16)), \
+            16, wsrc##SET[(q_) < WIW ? (q_) : 0], FR_KOFF_W(tile_), 0, 2);                                  \
+      else                                                                                                  \
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                           \
+            wrs##SET, (lptr_t)(lds_raw + (WBASE + (slot_) * C::WCH) * 16 + (((q_) / IW) * NW + vwi_) * (kWave * 16)), \
+            16, wsrc##SET[(q_) < WIW ? (q_) : 0], FR_KOFF_W(tile_), 0, 0);                                  \
     } else {                                                                                                \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                             \
           xrs##SET, (lptr_t)(lds_raw + (slot_) * (C::XCH * 16) + ((((q_) - WIW) / IW) * NW + vwi_) * (kWave * 16)), \
@@ -468,7 +478,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     /* vmcnt(0) once per tile: the previous tile's epilogue stores share the counter with the loads */     \
     FR_KTILE(ISS_, true, A, S, false, 0)                                                                   \
     FR_KTILE(ISS_, true, A, S + 1, false, (S - 2) * NLI)                                                   \
-    if (NEXT) FR_MAKE_SET(n_pid_t, n_pid_f, n_expert, n_kb, n_sid[ih], xsrcB, wsrcB, xrsB, wrsB)           \
+    if (NEXT) FR_MAKE_SET(n_pid_t, n_pid_f, n_expert, n_kb, n_sid[ih], xsrcB, wsrcB, xrsB, wrsB, ntB)      \
     __builtin_amdgcn_s_waitcnt(0xC07F); /* lgkmcnt(0): no scalar load pending inside the loops */          \
     for (int kt = 2; kt < kn - S; ++kt) FR_KTILE(ISS_, true, A, kt + S, false, (S - 2) * NLI)              \
     if (NEXT) {                                                                                            \
@@ -499,7 +509,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
     int unit = 0;                                                                                          \
     for (; unit + 1 < n_units; ++unit) { /* a next unit exists: hand the ring over to it */                \
       FR_TILE(ISS_, true)                                                                                  \
-      pid_t = n_pid_t; pid_f = n_pid_f; expert = n_expert; xrsA = xrsB; wrsA = wrsB;                       \
+      pid_t = n_pid_t; pid_f = n_pid_f; expert = n_expert; xrsA = xrsB; wrsA = wrsB; ntA = ntB;            \
       kb = n_kb; kn = n_kn; tu = n_tu;                                                                     \
       _Pragma("unroll") for (int ih = 0; ih < XIW; ++ih) xsrcA[ih] = xsrcB[ih];                        \
       _Pragma("unroll") for (int ih = 0; ih < WIW; ++ih) wsrcA[ih] = wsrcB[ih];                        \
