@@ -136,12 +136,12 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // With a 160-row candidate the 256-row tile takes over at 1200 pairs per expert (H >= 4096).  Below 112 pairs per expert one
   // block holds an expert either way and the smaller tile is cheaper (256 / 384 tokens: 548 / 556, 580 / 602 us);
   // with H = 1024 (16 K tiles) the 160-row tile loses (700 tokens: 85 / 96 us).
-  // fp8 (16x16x128 MFMAs for this tile; its gate/up kernel spills 46 registers): only where a fifth of the blocks
-  // go - 512 / 1024 tokens 435 / 392 and 543 / 505 us, but 2048 tokens 853 / 877 - and never instead of 256 rows
-  // (4096 tokens: 1506 against 1495 us).
+  // fp8 (16x16x128 MFMAs for this tile; its gate/up kernel spills 46 registers): only where a sixth of the blocks
+  // go - 128 / 160 / 256 rows: 512 tokens 435 / 392, 1024: 543 / 505, 2560: 1145 / 1006 / 1063 us, but 2048: 853 / 877
+  // / 899 - and below 900 pairs per expert (4096 tokens: 1506 against 1495 us with 256 rows).
   const bool two_byte = dtype == FR_BF16 || dtype == FR_F16;
-  if ((block == 128 || (block == 256 && two_byte)) && H >= 2048 && F >= 1024 && E <= 1022 && avg >= 112 &&
-      avg < (two_byte && H >= 4096 ? 1200.0 : t256)) {
+  if ((block == 128 || block == 256) && H >= 2048 && F >= 1024 && E <= 1022 && avg >= 112 &&
+      avg < (H >= 4096 ? (two_byte ? 1200.0 : 900.0) : t256)) {
     const double sigma = sqrt(avg * (1.0 - 1.0 / E)) + 1e-9;
     auto tail = [&](double x) { return 0.5 * erfc((x - avg) / (sigma * 1.4142135623730951)); };  // P(pairs of an expert > x)
     auto expected = [&](int rows) {  // expected multiples of `rows` that hold an expert's pairs

@@ -58,7 +58,7 @@ def test_plan_table():
     as documented (Mixtral shape: 16-row blocks up to 8 pairs per expert, 32 below 26, 64 below 52 at
     H >= 4096, then 128 or - where the spread of the experts' loads around a multiple of 128 would cost
     every other expert one block more - 160, 256 from 1200 pairs per expert on; fp8 takes 160 rows only where
-    a fifth of the blocks go and 256 from 560 on; the fine-grained shape with H = 2048 has no 64-row range and never
+    a sixth of the blocks go and 256 from 900 on; the fine-grained shape with H = 2048 has no 64-row range and never
     takes 256 rows below 4096 pairs per expert)."""
     from fast_route_amd import _native
     lib = _native.lib()
@@ -75,7 +75,8 @@ def test_plan_table():
     assert mix(1) == (16, 4) and mix(2) == (16, 2) and mix(3) == (16, 4) and mix(4) == (16, 4) and mix(16) == (16, 1)
     assert mix(128) == (64, 2)
     assert mix(4096)[1] == 1 and plan(16384, 4096, 14336, 8, 2)[0] == 256
-    assert [mix(M, _native.FR_FP8_E4M3)[0] for M in (103, 104, 207, 208, 512, 768, 1024, 2048, 2240)] == [32, 64, 64, 128, 160, 128, 160, 128, 256]
+    assert [mix(M, _native.FR_FP8_E4M3)[0] for M in (103, 104, 207, 208, 512, 768, 1024, 2048, 2560, 3600, 4096)] == \
+        [32, 64, 64, 128, 160, 128, 160, 128, 160, 256, 256]
     fine = lambda M: plan(M, 2048, 1408, 64, 6)[0]
     assert [fine(M) for M in (85, 86, 341, 342, 1246, 1247, 43690, 43691)] == [16, 32, 32, 128, 128, 160, 160, 256]
     # the scratch for splitting the last round exists exactly for 128- and 256-row blocks with a long K
