@@ -32,7 +32,7 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 SHAPES = {
-    "mixtral": dict(H=4096, F=14336, E=8, topk=2, zipf=False, sweep=[1, 16, 64, 256, 1024, 4096, 16384]),
+    "mixtral": dict(H=4096, F=14336, E=8, topk=2, zipf=False, sweep=[1, 16, 64, 256, 512, 1024, 2048, 4096, 16384]),
     "fine": dict(H=2048, F=1408, E=64, topk=6, zipf=True, sweep=[1, 32, 128, 512, 2048, 8192]),
     "small": dict(H=1024, F=3584, E=8, topk=2, zipf=False, sweep=[64]),
     "mixtral22b": dict(H=6144, F=16384, E=8, topk=2, zipf=False, sweep=[1, 16, 128, 1024, 4096]),
@@ -492,7 +492,7 @@ def other_configs(torch, N, args, mixtral_weights):
     w1, w2 = mixtral_weights
     fp8 = prepare_weights_fp8(w1, w2)
     sweep = []
-    for M in (16, 256, 4096):
+    for M in (16, 256, 1024, 4096):
         rec, layer = measure(torch, N, shape, M, w1, w2, steps, warmup, args.seed, fp8)
         sweep.append(dict(compact(rec), stage_us=rec["stage_us"]))
     out["fp8"] = {"workload": "Mixtral shape, e4m3 weights (scale per expert and output channel), bf16 activations quantised per token",
@@ -668,7 +668,7 @@ def main():
     if args.dtype == "fp8":
         from fast_route_amd import prepare_weights_fp8
         fp8 = prepare_weights_fp8(w1, w2)
-        sweep_ms = [16, 256, 4096] if args.shape == "mixtral" else shape["sweep"]
+        sweep_ms = [16, 256, 1024, 4096] if args.shape == "mixtral" else shape["sweep"]
     prepared = 0
     if args.prepared and fp8 is None:
         from fast_route_amd import prepare_weights
