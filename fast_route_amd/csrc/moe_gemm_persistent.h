@@ -179,9 +179,11 @@ __global__ __launch_bounds__(C::NT, C::MINB) void moe_gemm_persistent_kernel(con
   constexpr int ACC_N = (C::TILE == 32) ? 16 : 4;
   constexpr int S = C::STAGES, NW = C::NW, XIW = C::XIW, WIW = C::WIW, IW = C::IW, NLI = XIW + WIW;
   constexpr int NM = C::JF * C::IT, RD_AT = (NM + 1) / 2 - 1;
-  // one fragment buffer for fp8 (8-register fragments) and for the 256-row tile on 16x16 MFMAs (twelve fragments
-  // per K-step next to 128 accumulators), two otherwise
-  constexpr bool SINGLE = E::SCALED || (C::TILE == 16 && BT >= 256);
+  // one fragment buffer for fp8 (8-register fragments) and for the tiles on 16x16 MFMAs (nine to twelve fragments
+  // per K-step next to 64 to 128 accumulators: each fragment is read again as soon as its last MFMA of the K-step
+  // is issued; measured against two buffers: 256 rows needed it to fit, 160 rows -0.4 .. -1.3 %, 128 rows 0 .. -1 %),
+  // two otherwise
+  constexpr bool SINGLE = E::SCALED || C::TILE == 16;
   // fp8 epilogue: scales fetched up front where the registers allow it (the 256-row tile keeps 128 accumulators
   // and two address sets alive: measured 603 us with, 589 us without for the down projection at M = 4096; the
   // 128-row tile gains 2-5 %)
