@@ -267,7 +267,7 @@ def kernel_roofline(shape, rec, fp8=False):
     # blocks and for 256-row blocks of 2-byte operands, the plain tile kernel otherwise
     if not fp8 and M <= 4 and H >= 4096 and H % 512 == 0 and any(H // 512 % c == 0 for c in (5, 6, 7, 8)) and M * H * 2 <= 65536:
         name = "gateup_rows_kernel"
-    elif rec["block"] in (128, 160) or (rec["block"] == 256 and not fp8):
+    elif rec["block"] in (64, 128, 160) or (rec["block"] == 256 and not fp8):
         name = "moe_gemm_persistent_kernel<EPI_SILU>"
     else:
         name = "moe_gemm_kernel<EPI_SILU>"
