@@ -140,15 +140,15 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // go - 128 / 160 / 256 rows: 512 tokens 435 / 392, 1024: 543 / 505, 2560: 1145 / 1006 / 1063 us, but 2048: 853 / 877
   // / 899 - and below 900 pairs per expert (4096 tokens: 1506 against 1495 us with 256 rows).
   const bool two_byte = dtype == FR_BF16 || dtype == FR_F16;
+  const double sigma = sqrt(avg * (1.0 - 1.0 / E)) + 1e-9;  // spread of an expert's pairs under uniform routing
+  auto tail = [&](double x) { return 0.5 * erfc((x - avg) / (sigma * 1.4142135623730951)); };  // P(pairs of an expert > x)
+  auto expected = [&](int rows) {  // expected multiples of `rows` that hold an expert's pairs
+    double sum = 1.0;
+    for (int k = 1; k * rows < avg + 8 * sigma; ++k) sum += tail(static_cast<double>(k) * rows);
+    return sum;
+  };
   if ((block == 128 || block == 256) && H >= 2048 && F >= 1024 && E <= 1022 && avg >= 112 &&
       avg < (H >= 4096 ? (two_byte ? 1200.0 : 900.0) : t256)) {
-    const double sigma = sqrt(avg * (1.0 - 1.0 / E)) + 1e-9;
-    auto tail = [&](double x) { return 0.5 * erfc((x - avg) / (sigma * 1.4142135623730951)); };  // P(pairs of an expert > x)
-    auto expected = [&](int rows) {  // expected multiples of `rows` that hold an expert's pairs
-      double sum = 1.0;
-      for (int k = 1; k * rows < avg + 8 * sigma; ++k) sum += tail(static_cast<double>(k) * rows);
-      return sum;
-    };
     const double b128 = expected(128), b160 = expected(160);
     const double c128 = expected(64) * 64, c160 = expected(80) * 80;
     const bool take160 = two_byte ? (b160 * 1.15 < b128 || c160 <= 0.98 * c128) : b160 * 1.2 < b128;
@@ -159,7 +159,8 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   if (block == 160 && !two_byte && (H < 640 || F < 1024 || E > 1022)) block = 128;
   // Down projection: N = H gives few feature tiles, so K is split.
   const int bf = block == 16 ? 64 : (block == 32 ? 128 : 256);
-  const int64_t blocks = n <= E ? n : (block >= 128 ? ceil_div(n, block) + E / 2 : E);
+  // expected token blocks: one per pair or per expert in the decode regime, else the expected blocks per expert
+  const int64_t blocks = n <= E ? n : (block >= 128 ? static_cast<int64_t>(E * expected(block) + 0.5) : E);
   const int64_t tiles = blocks * ceil_div(H, bf);
   const int bk_elems = dtype == FR_FP8_E4M3 ? (block <= 32 ? 256 : 128) : (block == 16 ? 128 : 64);
   // 256-row tiles of 2-byte operands with a long K balance their last round themselves (its
@@ -170,16 +171,20 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
     // whole rounds plus a split last round, or so few tiles that every one is cut into 4..8 slices;
     // in between (most of one round: no idle workgroups to cut for) all tiles are split alike
   } else if (block >= 128) {
-    // one workgroup per CU: the split that minimises GEMM time (how well tiles x split fill whole rounds
-    // of 256 CUs, at ~0.9 PFLOP/s) plus the partial traffic it causes (one 2-byte slice, or `split` fp32
-    // slices, written and read back at ~4 TB/s: with many pairs per weight byte that traffic decides)
+    // one workgroup per CU: the split that minimises GEMM time (at ~0.9 PFLOP/s, stretched by how long the
+    // busiest workgroup works: the persistent launch gives each of `sp` slices 256 / sp workgroups, rounded down
+    // to whole XCD shares, and a workgroup does ceil(tiles / those) units of 1 / sp of a tile) plus the partial
+    // traffic it causes (one 2-byte slice, or `split` fp32 slices, written and read back at ~4 TB/s: with many
+    // pairs per weight byte that traffic decides).  Measured on 8 experts with one block each (128 tiles), down
+    // projection with 1 / 2 / 3 / 4 slices: 384 tokens 185 / 174 / 212 / 196 us, 512 tokens 202 / 194 / 233 / 214.
     double best = 1e30;
     const double rows = static_cast<double>(blocks) * block, pairs = static_cast<double>(n);
     for (int sp = 1; sp <= 4; ++sp) {
       if (F / sp < 8 * bk_elems) break;
-      const double work = static_cast<double>(tiles) * sp;
-      const double fill = work / (256.0 * static_cast<double>(ceil_div(tiles * sp, 256)));
-      const double t_gemm = 2.0 * rows * H * F / 0.9e15 / fill;
+      const int64_t wgs = 256 / sp / 8 * 8;
+      const double busiest = static_cast<double>(ceil_div(tiles, wgs)) / sp;  // in tiles
+      const double fill = (static_cast<double>(tiles) / 256.0) / busiest;
+      const double t_gemm = 2.0 * rows * H * F / 0.9e15 / (fill < 1.0 ? fill : 1.0);
       const double t_part = pairs * H * (sp == 1 ? 2.0 : 4.0 * sp) * 2.0 / 4e12;
       if (t_gemm + t_part < best) { best = t_gemm + t_part; split = sp; }
     }
