@@ -218,7 +218,24 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_rsrc(const T* p, unsig
 }
 #endif
 
-template <typename T, typename C, int EPI, bool HOIST = true, typename AccT>
+#if defined(__HIP_DEVICE_COMPILE__)
+// The four registers of an accumulator tile that lives in the accumulation half of the register file, copied to
+// ordinary registers here and now.  (Left to itself the register allocator moves every accumulator to an ordinary
+// register right behind its last MFMA - a wait for the MFMA's result each, and 256 values that do not fit.)
+__device__ __forceinline__ f32x4 acc_fetch(const f32x4& v) {
+  f32x4 o;
+  asm volatile("v_accvgpr_read_b32 %0, %4\n\tv_accvgpr_read_b32 %1, %5\n\tv_accvgpr_read_b32 %2, %6\n\tv_accvgpr_read_b32 %3, %7"
+               : "=v"(o[0]), "=v"(o[1]), "=v"(o[2]), "=v"(o[3])
+               : "a"(v[0]), "a"(v[1]), "a"(v[2]), "a"(v[3]));
+  return o;
+}
+#else
+__device__ __forceinline__ f32x4 acc_fetch(const f32x4& v) { return v; }
+#endif
+__device__ __forceinline__ f32x16 acc_fetch(const f32x16& v) { return v; }
+
+// AG: the accumulators live in the accumulation registers (one wavefront per SIMD) and are fetched tile by tile.
+template <typename T, typename C, int EPI, bool HOIST = true, bool AG = false, typename AccT>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::JF][C::IT], int pid_t, int pid_f,
                                               int expert, int split, int wt, int wf, int frow, int kgrp) {
   typedef Elem<T> E;
@@ -231,6 +248,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
   // group g (TILE==32: 4 groups of 4 regs; TILE==16: one), 4 consecutive features
   // starting at g*8 + kgrp*4 (TILE==32) or kgrp*4 (TILE==16) inside the MFMA tile.
   constexpr int GROUPS = ACC_N / 4;
+  // accumulators in the accumulation registers: results are fetched, computed and stored group by group
+  constexpr bool kFence = AG;
   // fp8: with HOIST the scales of the lane's weight rows (the same for every token tile) and of its token rows
   // are fetched up front, all loads in flight together, instead of one by one between the stores (which the
   // compiler may not move them across).  That takes JF * ACC_N registers: the persistent kernel, which keeps
@@ -303,9 +322,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
         for (int g = 0; g < GROUPS; ++g) {
           const int f = pid_f * (BF / 2) + wf * (C::TF / 2) + j * C::TILE + g * 8 + kgrp * 4;
           out4 o;
+          const AccT ga = AG ? acc_fetch(acc[j][i]) : acc[j][i], ua = AG ? acc_fetch(acc[j + HJ][i]) : acc[j + HJ][i];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            float gv = acc[j][i][g * 4 + r], uv = acc[j + HJ][i][g * 4 + r];
+            float gv = ga[g * 4 + r], uv = ua[g * 4 + r];
             if constexpr (E::SCALED) {
               gv *= xs * w_scale(j, g, r);
               uv *= xs * w_scale(j + HJ, g, r);
@@ -316,6 +336,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
           else
             for (int r = 0; r < 4; ++r)
               if (f + r < a.N) orow[f + r] = o[r];
+          if constexpr (kFence) __builtin_amdgcn_sched_barrier(0);
         }
     } else {
       if (sid < a.num_valid) {
@@ -326,9 +347,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
           for (int g = 0; g < GROUPS; ++g) {
             const int f = pid_f * BF + wf * C::TF + j * C::TILE + g * 8 + kgrp * 4;
             float v[4];
+            const AccT ca = AG ? acc_fetch(acc[j][i]) : acc[j][i];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              v[r] = acc[j][i][g * 4 + r] * rw;
+              v[r] = ca[g * 4 + r] * rw;
               if constexpr (E::SCALED) v[r] *= w_scale(j, g, r);
             }
             if constexpr (EPI == EPI_DOWN) {
@@ -353,6 +375,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
                     if (f + r < a.N) orow[f + r] = o[r];
               }
             }
+            if constexpr (kFence) __builtin_amdgcn_sched_barrier(0);
           }
       }
     }

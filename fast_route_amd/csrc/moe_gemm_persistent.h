@@ -101,13 +101,19 @@ __device__ __forceinline__ void expert_block_offsets(const GemmArgs& a, int nt, 
     if (a.expert_ids[b] < a.expert_ids[b - 1]) off[kMaxExperts + 1] = 1;
   __syncthreads();
 }
+// A tile's place among the tiles that share its weight tile: the `count` token blocks of its chunk, of which it
+// is number `index` (1 and 0 without a walk table).
+struct TileShare {
+  int count, index;
+};
 __device__ __forceinline__ void tile_coords(const GemmArgs& a, const int* off, int lin, int& pid_t, int& pid_f,
-                                            int& expert) {
+                                            int& expert, TileShare* share = nullptr) {
   const int F = a.num_f_tiles;
   if (off[kMaxExperts + 1]) {
     pid_t = lin / F;
     pid_f = lin % F;
     expert = a.expert_ids[pid_t];
+    if (share) *share = TileShare{1, 0};
     return;
   }
   expert = a.expert_ids[lin / F];  // lin / F is one of the expert's blocks: its tiles are [off[e] * F, off[e + 1] * F)
@@ -130,6 +136,7 @@ __device__ __forceinline__ void tile_coords(const GemmArgs& a, const int* off, i
   }
   pid_t = start + q % gsz;
   pid_f = q / gsz;
+  if (share) *share = TileShare{gsz, q % gsz};
 }
 // Tile column of accumulator tile j of feature wavefront wf (= row of the weight tile in LDS).
 template <typename C, int EPI>
@@ -142,19 +149,22 @@ __device__ __forceinline__ int acc_tile_col(int wf, int j) {
   }
 }
 // fp32 accumulators of one K slice, as they are, to the slice's [BT][BF] buffer
-template <typename C, int EPI, typename AccT>
+template <typename C, int EPI, bool AG = false, typename AccT>
 __device__ __forceinline__ void tail_store(float* tile, AccT (&acc)[C::JF][C::IT], int wt, int wf, int frow, int kgrp) {
   constexpr int GROUPS = ((C::TILE == 32) ? 16 : 4) / 4;
 #pragma unroll
   for (int i = 0; i < C::IT; ++i) {
     float* row = tile + (wt * C::TT + i * C::TILE + frow) * C::BF;
 #pragma unroll
-    for (int j = 0; j < C::JF; ++j)
+    for (int j = 0; j < C::JF; ++j) {
+      const AccT ca = AG ? acc_fetch(acc[j][i]) : acc[j][i];
 #pragma unroll
       for (int g = 0; g < GROUPS; ++g) {
-        const f32x4 o = {acc[j][i][g * 4 + 0], acc[j][i][g * 4 + 1], acc[j][i][g * 4 + 2], acc[j][i][g * 4 + 3]};
+        const f32x4 o = {ca[g * 4 + 0], ca[g * 4 + 1], ca[g * 4 + 2], ca[g * 4 + 3]};
         *reinterpret_cast<f32x4*>(row + acc_tile_col<C, EPI>(wf, j) + g * 8 + kgrp * 4) = o;
+        if constexpr (AG) __builtin_amdgcn_sched_barrier(0);
       }
+    }
   }
 }
 

@@ -3,7 +3,7 @@
 // (moe_gemm_inst_*.hip) so that the library builds in parallel; moe_gemm.hip sees only
 // the declaration of dispatch_block.
 #pragma once
-#include "moe_gemm_persistent.h"
+#include "moe_gemm_quad.h"
 
 namespace fr {
 
@@ -90,6 +90,13 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       else {
         // 2-byte operands, long K: the 16x16x32 MFMA form (see Tiles::T256S)
         if constexpr (sizeof(T) == 2) {
+          // one wavefront per SIMD, 128 x 128 outputs each (see moe_gemm_quad.h), where its K loop is long enough
+#ifndef FR_NO_QUAD
+          {
+            const int rc = launch_gemm_quad<T, EPI>(a, splits, st);
+            if (rc != 1) return rc;
+          }
+#endif
           if (a.K >= kSmallMfmaMinK) return launch_gemm_persistent<T, typename TL::T256S, EPI>(a, splits, st);
         }
         return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
@@ -146,6 +153,7 @@ int prepare_tiles() {
   int rc = launch_gemm_persistent<T, typename TL::T256, EPI>(a, 1, nullptr);
   if constexpr (sizeof(T) == 2) {
     if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T256S, EPI>(a, 1, nullptr);
+    if (rc == FR_OK) rc = launch_gemm_quad<T, EPI>(a, 1, nullptr);
   }
   if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T128P, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T160P, EPI>(a, 1, nullptr);
