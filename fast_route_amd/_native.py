@@ -22,7 +22,7 @@ class FrMoePlan(ctypes.Structure):
 
 class FrMoeTunables(ctypes.Structure):
     _fields_ = [("block", c_int32), ("split_k", c_int32), ("group_m", c_int32), ("no_tail_split", c_int32),
-                ("epilogue_combine", c_int32)]
+                ("epilogue_combine", c_int32), ("no_quad", c_int32)]
 
 
 # name -> (restype, argtypes); must list every symbol the header declares

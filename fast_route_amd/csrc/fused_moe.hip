@@ -77,7 +77,7 @@ using namespace fr;
 
 extern "C" int fr_moe_set_tunables(const fr_moe_tunables* t) {
   if (!t) {
-    g_tunables = fr_moe_tunables{0, 0, 0, 0, 0};
+    g_tunables = fr_moe_tunables{0, 0, 0, 0, 0, 0};
     return FR_OK;
   }
   FR_REQUIRE(t->block == 0 || t->block == 16 || t->block == 32 || t->block == 64 || t->block == 128 || t->block == 160 || t->block == 256,
@@ -86,6 +86,7 @@ extern "C" int fr_moe_set_tunables(const fr_moe_tunables* t) {
   FR_REQUIRE(t->group_m >= 0 && t->group_m <= 64, FR_E_SHAPE, "fr_moe_set_tunables: group_m=%d outside [0, 64]", t->group_m);
   FR_REQUIRE(t->no_tail_split == 0 || t->no_tail_split == 1, FR_E_SHAPE, "fr_moe_set_tunables: no_tail_split=%d", t->no_tail_split);
   FR_REQUIRE(t->epilogue_combine == 0 || t->epilogue_combine == 1, FR_E_SHAPE, "fr_moe_set_tunables: epilogue_combine=%d", t->epilogue_combine);
+  FR_REQUIRE(t->no_quad == 0 || t->no_quad == 1, FR_E_SHAPE, "fr_moe_set_tunables: no_quad=%d", t->no_quad);
   g_tunables = *t;
   return FR_OK;
 }
@@ -153,6 +154,19 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
     const double c128 = expected(64) * 64, c160 = expected(80) * 80;
     const bool take160 = two_byte ? (b160 * 1.15 < b128 || c160 <= 0.98 * c128) : b160 * 1.2 < b128;
     if (take160) block = 160;
+  }
+  // 256 rows on the one-wavefront-per-SIMD kernel (2-byte operands, 16 K tiles or more in both GEMMs): a row of its
+  // tiles costs about 8 % less than one of the 128- or 160-row tiles (4096 tokens 2365 against 2510 us with 160 rows,
+  // 16384: 8494 / 9349), which pays wherever its coarser blocks do not add more rows than that.  Its rows: the mean
+  // of whole blocks (the time of a tile) and whole half blocks (the wavefronts of an all-padding half idle: energy,
+  // and the clock follows the energy).  Measured 160 / 256 rows on 8 experts, H = 4096: 1280 tokens 982 / 1040 us
+  // (160 stays), 1536: 1148 / 1081, 1792: 1216 / 1102, 2048: 1395 / 1373, 2304: 1490 / 1626 (160 stays), 2560:
+  // 1664 / 1647, 3072: 1973 / 1815, 5120: 3059 / 2911, 8192: 4804 / 4339.  Below 350 pairs per expert the smaller
+  // tiles stream the weights faster (1024 tokens: 811 / 977 us).
+  if (two_byte && !g_tunables.no_quad && (block == 128 || block == 160) && H >= 4096 && F >= 1024 && E <= 1022 && avg >= 350) {
+    const double other = expected(block) * block;
+    const double quad = 0.5 * (expected(256) * 256 + expected(128) * 128);
+    if (quad <= 1.08 * other) block = 256;
   }
   if (g_tunables.block) block = g_tunables.block;
   // the fp8 160-row tile exists in the persistent form only (five K tiles per K slice at least, 1022 experts at most)

@@ -38,6 +38,27 @@ constexpr int kQuadMinTiles = 8;    // K tiles per work unit, at least (two peel
 constexpr int kQuadTouchAhead = FQ_AHEAD;  // K tiles between a touch and the tile loads of the same rows
 constexpr int kQuadSink = 1024;     // bytes of LDS the touches land in (256 per wavefront)
 
+#ifndef FQ_RD0
+#define FQ_RD0 3
+#endif
+#ifndef FQ_RD1
+#define FQ_RD1 4
+#endif
+#ifndef FQ_LD_POS
+#define FQ_LD_POS 2
+#endif
+#ifndef FQ_LD_EVERY
+#define FQ_LD_EVERY 4
+#endif
+#ifndef FQ_TOUCH_AT
+#define FQ_TOUCH_AT 63
+#endif
+#ifndef FQ_XSHARE
+#define FQ_XSHARE 4
+#endif
+#ifndef FQ_PRIO
+#define FQ_PRIO 0
+#endif
 #ifndef FQ_TOUCH
 #define FQ_TOUCH 1
 #endif
@@ -54,9 +75,9 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
   constexpr int NM = NF * NF;                 // MFMAs per K-step
   constexpr int NW = 4, XI = 8, WI = 8, NL = XI + WI;  // tile loads per wavefront and K tile
   constexpr int XBYTES = C::XCH * 16, WBYTES = C::WCH * 16, SLOT = XBYTES + WBYTES;  // a ring slot: X rows, then W rows
-  constexpr int RD0 = 3, RD1 = 4;             // one fragment read after every n-th MFMA of the first / second K-step
-  constexpr int LD_POS = 2, LD_EVERY = 4;     // tile load q after MFMA LD_POS + q * LD_EVERY of the second K-step
-  constexpr int TOUCH_AT = NM - 1;
+  constexpr int RD0 = FQ_RD0, RD1 = FQ_RD1;   // one fragment read after every n-th MFMA of the first / second K-step
+  constexpr int LD_POS = FQ_LD_POS, LD_EVERY = FQ_LD_EVERY;  // tile load q after MFMA LD_POS + q * LD_EVERY of the second K-step
+  constexpr int TOUCH_AT = FQ_TOUCH_AT;
   static_assert(C::IT == NF && C::JF == NF && C::XIW == XI && C::WIW == WI && C::KGROUPS == 4 && CPR == 8, "128 x 128 per wavefront");
   static_assert(LD_POS + (NL - 1) * LD_EVERY < NM && 15 * RD0 < NM && 15 * RD1 < NM, "loads and reads fit their K-step");
 
@@ -142,7 +163,7 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
     const int cnt_ = max(1, min((sh_).count, 32));                                             \
     const int per_ = (BF + cnt_ - 1) / cnt_, pw_ = (per_ + NW - 1) / NW;                       \
     wrow_ = min((sh_).index * per_ + wave_u * pw_ + (lane < pw_ ? lane : 0), BF - 1);          \
-    const int xs_ = max(1, min(4, 32 / cnt_)), xper_ = BT / xs_, xw_ = xper_ / NW;             \
+    const int xs_ = max(1, min(FQ_XSHARE, 32 / cnt_)), xper_ = BT / xs_, xw_ = xper_ / NW;             \
     xrow_ = ((pf_) % xs_) * xper_ + wave_u * xw_ + (lane < xw_ ? lane : 0);                    \
     xon_ = lane < xw_;                                                                         \
   }

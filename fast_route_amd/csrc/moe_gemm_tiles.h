@@ -91,12 +91,10 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
         // 2-byte operands, long K: the 16x16x32 MFMA form (see Tiles::T256S)
         if constexpr (sizeof(T) == 2) {
           // one wavefront per SIMD, 128 x 128 outputs each (see moe_gemm_quad.h), where its K loop is long enough
-#ifndef FR_NO_QUAD
-          {
+          if (!tunables().no_quad) {
             const int rc = launch_gemm_quad<T, EPI>(a, splits, st);
             if (rc != 1) return rc;
           }
-#endif
           if (a.K >= kSmallMfmaMinK) return launch_gemm_persistent<T, typename TL::T256S, EPI>(a, splits, st);
         }
         return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);

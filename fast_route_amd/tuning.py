@@ -13,12 +13,14 @@ from . import _native as N
 
 
 def set_tunables(block: int = 0, split_k: int = 0, group_m: int = 0, no_tail_split: bool = False,
-                 epilogue_combine: bool = False) -> None:
+                 epilogue_combine: bool = False, no_quad: bool = False) -> None:
     """0 leaves a choice to the library.  block: routing block / token rows per tile
     (16, 32, 64, 128, 160, 256); split_k: K slices of the down projection; group_m: token blocks
     walked together over the feature tiles; no_tail_split: never split the last round of tiles;
-    epilogue_combine: top-2 combine by atomic adds in the down GEMM's epilogue (measured slower than the combine kernel)."""
-    t = N.FrMoeTunables(int(block), int(split_k), int(group_m), int(bool(no_tail_split)), int(bool(epilogue_combine)))
+    epilogue_combine: top-2 combine by atomic adds in the down GEMM's epilogue (measured slower than the combine kernel);
+    no_quad: 256-row tiles take the eight-wavefront kernel instead of the one-wavefront-per-SIMD one (same results)."""
+    t = N.FrMoeTunables(int(block), int(split_k), int(group_m), int(bool(no_tail_split)), int(bool(epilogue_combine)),
+                        int(bool(no_quad)))
     N.check(N.lib().fr_moe_set_tunables(ctypes.byref(t)))
 
 
@@ -30,7 +32,7 @@ def get_tunables() -> dict:
     t = N.FrMoeTunables()
     N.check(N.lib().fr_moe_get_tunables(ctypes.byref(t)))
     return {"block": t.block, "split_k": t.split_k, "group_m": t.group_m, "no_tail_split": bool(t.no_tail_split),
-            "epilogue_combine": bool(t.epilogue_combine)}
+            "epilogue_combine": bool(t.epilogue_combine), "no_quad": bool(t.no_quad)}
 
 
 @contextlib.contextmanager

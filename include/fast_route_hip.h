@@ -167,6 +167,9 @@ int fr_moe_prepare(int dtype);
  *              combine kernel.  Off by default: measured slower - 16.7 M four-byte atomics at Mixtral
  *              shape and 4096 tokens cost the down stage 1015 us against 900 us (3650 against 3200 us at
  *              16384 tokens, 149 against 146 us at 16 tokens)
+ *   no_quad    1: 256-row tiles of 2-byte operands never take the one-wavefront-per-SIMD kernel
+ *              (four wavefronts of 128 x 128 outputs, the default where K has 16 K tiles or more) but the
+ *              eight-wavefront one; same results bit for bit, for comparisons and tests
  * fr_moe_get_plan, fr_fused_moe, fr_fused_experts, fr_fused_moe_fp8 and the staged GEMM entry
  * points all see them.  fr_moe_set_tunables(NULL) restores the defaults.
  * The staged entry points read the knobs when they are called, not when the plan was made: a
@@ -184,6 +187,7 @@ typedef struct fr_moe_tunables {
   int32_t group_m;
   int32_t no_tail_split;
   int32_t epilogue_combine;
+  int32_t no_quad;
 } fr_moe_tunables;
 int fr_moe_set_tunables(const fr_moe_tunables* t);
 int fr_moe_get_tunables(fr_moe_tunables* t);

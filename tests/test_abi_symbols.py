@@ -57,7 +57,8 @@ def test_plan_table():
     """The tile plan is host logic: routing block and K slices of the down projection per token count,
     as documented (Mixtral shape: 16-row blocks up to 8 pairs per expert, 32 below 26, 64 below 52 at
     H >= 4096, then 128 or - where the spread of the experts' loads around a multiple of 128 would cost
-    every other expert one block more - 160, 256 from 1200 pairs per expert on; fp8 takes 160 rows only where
+    every other expert one block more - 160; 2-byte operands take 256 rows (one wavefront per SIMD) from 350 pairs
+    per expert on wherever their coarser blocks add less than 8 % of rows, 256 from 1200 pairs on otherwise; fp8 takes 160 rows only where
     a sixth of the blocks go and 256 from 900 on; the fine-grained shape with H = 2048 has no 64-row range and never
     takes 256 rows below 4096 pairs per expert)."""
     from fast_route_amd import _native
@@ -70,8 +71,15 @@ def test_plan_table():
         return p.block, p.split_k
 
     mix = lambda M, dt=_native.FR_BF16: plan(M, 4096, 14336, 8, 2, dt)
-    assert [mix(M)[0] for M in (1, 32, 33, 103, 104, 207, 208, 469, 470, 670, 671, 768, 1024, 2048, 4096, 4799, 4800)] == \
-        [16, 16, 32, 32, 64, 64, 128, 128, 160, 160, 128, 128, 160, 128, 160, 160, 256]
+    assert [mix(M)[0] for M in (1, 32, 33, 103, 104, 207, 208, 469, 470, 670, 671, 768, 1024, 1280, 1400, 1536, 2048, 2304, 2560,
+                               4096, 4800)] == \
+        [16, 16, 32, 32, 64, 64, 128, 128, 160, 160, 128, 128, 160, 160, 128, 256, 256, 160, 256, 256, 256]
+    import fast_route_amd as fr
+    try:  # without the one-wavefront-per-SIMD kernel the 256-row tile takes over at 1200 pairs per expert
+        with fr.tunables(no_quad=True):
+            assert [mix(M)[0] for M in (1536, 2048, 4096, 4799, 4800)] == [160, 128, 160, 160, 256]
+    finally:
+        fr.reset_tunables()
     assert mix(1) == (16, 4) and mix(2) == (16, 2) and mix(3) == (16, 4) and mix(4) == (16, 4) and mix(16) == (16, 1)
     assert mix(128) == (64, 2)
     assert mix(4096)[1] == 1 and plan(16384, 4096, 14336, 8, 2)[0] == 256
@@ -156,14 +164,14 @@ def test_tunables_override_the_plan_and_reset():
         return p
 
     base = plan(4096)
-    assert (base.block, base.split_k) == (160, 1) and base.tail_bytes > 0
+    assert (base.block, base.split_k) == (256, 1) and base.tail_bytes > 0
     try:
         fr.set_tunables(block=128, split_k=3)
         p = plan(4096)
         assert (p.block, p.split_k) == (128, 3) and p.sorted_len == 8192 + 8 * 127
-        assert fr.get_tunables() == {"block": 128, "split_k": 3, "group_m": 0, "no_tail_split": False, "epilogue_combine": False}
+        assert fr.get_tunables() == {"block": 128, "split_k": 3, "group_m": 0, "no_tail_split": False, "epilogue_combine": False, "no_quad": False}
         with fr.tunables(no_tail_split=True):
-            assert plan(4096).tail_bytes == 0 and plan(4096).block == 160  # the context replaces, then restores
+            assert plan(4096).tail_bytes == 0 and plan(4096).block == 256  # the context replaces, then restores
         assert plan(4096).block == 128
         fr.set_tunables(split_k=64)  # as many slices as keep 8 K tiles each: 14336 / (8 * 64) = 28
         assert plan(4096).split_k == 28

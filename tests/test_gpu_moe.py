@@ -656,6 +656,49 @@ def test_persistent_tiles_alternating_half_empty_and_full_blocks(native, block, 
         fr.reset_tunables()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_one_wavefront_per_simd_tile_equals_the_eight_wavefront_tile(native, dtype):
+    """256-row blocks with 16 K tiles or more run on four wavefronts of 128 x 128 outputs (moe_gemm_quad_kernel);
+    the no_quad knob sends the same call to the eight-wavefront kernel.  Same MFMA shape and K order: outputs equal
+    bit for bit, and both match the oracle.  64 experts with a seeded mix of full, under-half and over-half blocks,
+    16 / 8 feature tiles: every workgroup walks several units (hand-over of the ring), meets all-padding halves,
+    and the last round of tiles is split along K (32 K tiles in the gate/up GEMM)."""
+    import fast_route_amd as fr
+    from fast_route_amd import fused_experts, fused_moe
+    E, H, Fd = 64, 2048, 2048
+    rng = np.random.default_rng(5)
+    counts = np.where(rng.random(E) < 0.4, 256, rng.integers(1, 200, E))
+    ids = torch.from_numpy(np.repeat(np.arange(E), counts)).int()
+    ids = ids[torch.from_numpy(rng.permutation(ids.numel()))].view(-1, 1)
+    M = ids.shape[0]
+    _say(f"quad tile vs eight-wavefront tile {dtype} M={M}")
+    x, _, w1, w2 = _inputs(M, H, Fd, E, 77, dtype)
+    wts = torch.rand(M, 1) + 0.5
+    xd, w1d, w2d, wd, idd = x.cuda(), w1.cuda(), w2.cuda(), wts.cuda(), ids.cuda()
+    try:
+        with fr.tunables(block=256):
+            quad = fused_experts(xd, w1d, w2d, wd, idd)
+        with fr.tunables(block=256, no_quad=True):
+            eight = fused_experts(xd, w1d, w2d, wd, idd)
+        with fr.tunables(block=256, no_tail_split=True):
+            whole = fused_experts(xd, w1d, w2d, wd, idd)
+        torch.cuda.synchronize()
+        assert torch.equal(quad, eight), "the two 256-row kernels differ"
+        _assert_close(quad, oracle.moe_experts(x, w1, w2, wts, ids), dtype, "quad tile, experts only")
+        _assert_close(whole, oracle.moe_experts(x, w1, w2, wts, ids), dtype, "quad tile, no tail split")
+        # the layer with gating: top-2 of 8 experts, token rows gathered by sorted id, padding rows not fetched
+        x2, logits, w1b, w2b = _inputs(1500, 1024, 1024, 8, 78, dtype)
+        with fr.tunables(block=256):
+            a = fused_moe(x2.cuda(), w1b.cuda(), w2b.cuda(), logits.cuda(), 2, True)
+        with fr.tunables(block=256, no_quad=True):
+            b = fused_moe(x2.cuda(), w1b.cuda(), w2b.cuda(), logits.cuda(), 2, True)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), "the two 256-row kernels differ (layer with gating)"
+        _assert_close(a, oracle.fused_moe(x2, w1b, w2b, logits, 2, True), dtype, "quad tile, layer")
+    finally:
+        fr.reset_tunables()
+
+
 @pytest.mark.parametrize("E,k,H", [(8, 2, 4096), (64, 6, 4096), (100, 3, 4096), (256, 8, 4096), (4, 4, 4096), (16, 1, 4096),
                                    (64, 6, 2048), (8, 2, 3072), (16, 4, 2560)])
 @pytest.mark.parametrize("ldtype", [torch.float32, torch.bfloat16])
