@@ -31,6 +31,7 @@
 namespace fr {
 
 typedef Cfg<256, 256, 128, 2, 2, 16, 1, 2, 0, 1> QuadCfg;
+typedef Cfg<128, 256, 128, 1, 4, 16, 1, 2, 0, 1> QuadHalfCfg;  // output geometry of a half tile: 128 rows, a quarter of the features per wavefront
 constexpr int kQuadMinTiles = 8;    // K tiles per work unit, at least (two peeled at each end, the touch distance)
 #ifndef FQ_AHEAD
 #define FQ_AHEAD 3
@@ -59,6 +60,9 @@ constexpr int kQuadSink = 1024;     // bytes of LDS the touches land in (256 per
 #ifndef FQ_PRIO
 #define FQ_PRIO 0
 #endif
+#ifndef FQ_HALF
+#define FQ_HALF 1
+#endif
 #ifndef FQ_TOUCH
 #define FQ_TOUCH 1
 #endif
@@ -67,6 +71,7 @@ template <typename T, int EPI>
 __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a FR_PROF_PARAM) {
 #if defined(__HIP_DEVICE_COMPILE__)
   typedef QuadCfg C;
+  typedef QuadHalfCfg CH;
   typedef Elem<T> E;
   typedef __attribute__((address_space(3))) void* lptr_t;
   static_assert(sizeof(T) == 2, "2-byte operands");
@@ -77,9 +82,7 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
   constexpr int XBYTES = C::XCH * 16, WBYTES = C::WCH * 16, SLOT = XBYTES + WBYTES;  // a ring slot: X rows, then W rows
   constexpr int RD0 = FQ_RD0, RD1 = FQ_RD1;   // one fragment read after every n-th MFMA of the first / second K-step
   constexpr int LD_POS = FQ_LD_POS, LD_EVERY = FQ_LD_EVERY;  // tile load q after MFMA LD_POS + q * LD_EVERY of the second K-step
-  constexpr int TOUCH_AT = FQ_TOUCH_AT;
   static_assert(C::IT == NF && C::JF == NF && C::XIW == XI && C::WIW == WI && C::KGROUPS == 4 && CPR == 8, "128 x 128 per wavefront");
-  static_assert(LD_POS + (NL - 1) * LD_EVERY < NM && 15 * RD0 < NM && 15 * RD1 < NM, "loads and reads fit their K-step");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 
@@ -131,17 +134,24 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
   };
 
   // ---- fragment addresses: one per operand and K-step, the fragments at immediate offsets ------
+  // Whole tile: wavefront (wt, wf) owns token rows [wt * 128, + 128) x the weight rows acc_tile_col<C>(wf, .).
+  // Half tile (the block's upper 128 slots are all padding): wavefront w owns token rows [0, 128) x the weight
+  // rows acc_tile_col<CH>(w, .) - a quarter of the features each, so that the four MFMA pipes share what is left.
+  // All of a lane's fragment rows lie multiples of 16 apart (one swizzle key), and the two forms differ by
+  // wavefront-uniform distances.
   const int frow = lane & 15, kgrp = lane >> 4;
-  const int xrow0 = wt * C::TT + frow, wrow0 = acc_tile_col<C, EPI>(wf, 0) + frow;
-  const int xkey0 = swizzle<CPR>(xrow0, 0), wkey0 = swizzle<CPR>(wrow0, 0);
-  int xadr[2], wadr[2];  // byte addresses in slot 0
+  const int key0 = swizzle<CPR>(frow, 0);
+  int xadr[2], wadr[2];  // byte addresses in slot 0 of the fragments of row frow of the X tile / the W tile
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
-    xadr[s] = (xrow0 * CPR + ((s * 4 + kgrp) ^ xkey0)) * 16;
-    wadr[s] = XBYTES + (wrow0 * CPR + ((s * 4 + kgrp) ^ wkey0)) * 16;
+    xadr[s] = (frow * CPR + ((s * 4 + kgrp) ^ key0)) * 16;
+    wadr[s] = XBYTES + xadr[s];
   }
+  const int xbaseF = wt * C::TT * CPR * 16, wbaseF = acc_tile_col<C, EPI>(wf, 0) * CPR * 16;
+  const int wbaseH = acc_tile_col<CH, EPI>(wave_u, 0) * CPR * 16;
 #define FQ_XD(i_) ((i_) * 16 * CPR * 16)
-#define FQ_WD(j_) ((acc_tile_col<C, EPI>(0, (j_)) - acc_tile_col<C, EPI>(0, 0)) * CPR * 16)
+#define FQ_WD(HALF, j_) ((HALF) ? (acc_tile_col<CH, EPI>(0, (j_)) - acc_tile_col<CH, EPI>(0, 0)) * CPR * 16 \
+                               : (acc_tile_col<C, EPI>(0, (j_)) - acc_tile_col<C, EPI>(0, 0)) * CPR * 16)
 
   f32x4 acc[NF][NF];
   u32x4 fw[2][NF], fx[2][NF];
@@ -149,24 +159,32 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
   // ---- address sets: A = unit being multiplied, B = the workgroup's next unit ---------------------
   int pid_t, pid_f, expert, kb, kn, tu;
   int n_pid_t = 0, n_pid_f = 0, n_expert = 0, n_kb = 0, n_kn = 0, n_tu = -1;
+  bool half = false, n_half = false;  // the unit is a half tile
   TileShare shA, shB;
-  int n_sid[XI], n_tsid = 0;
+  int n_sid[XI], n_tsid = 0, n_up0 = 0, n_up1 = 0;
   unsigned xsrcA[XI], wsrcA[WI], xsrcB[XI], wsrcB[WI];
   unsigned twA = 0, txA = 0, twB = 0, txB = 0;  // touch offsets (weight rows, token rows) of this lane
   __amdgpu_buffer_rsrc_t xrsA, wrsA, xrsB, wrsB;
   // Touch shares.  Weight K tile (256 rows): shared by the sh.count token blocks of the tile's chunk, block
   // sh.index asks for rows [index * per, + per), per = ceil(256 / count), a quarter of them per wavefront.
   // Token K tile (256 gathered rows): shared by the feature tiles of the block an XCD holds at one time, about
-  // 32 / count of them, at most 4: feature tile f asks for share f % that many.
+  // 32 / count of them, at most FQ_XSHARE: feature tile f asks for share f % that many.
 #define FQ_TOUCH_ROWS(sh_, pf_, wrow_, xrow_, xon_)                                            \
   {                                                                                            \
     const int cnt_ = max(1, min((sh_).count, 32));                                             \
     const int per_ = (BF + cnt_ - 1) / cnt_, pw_ = (per_ + NW - 1) / NW;                       \
     wrow_ = min((sh_).index * per_ + wave_u * pw_ + (lane < pw_ ? lane : 0), BF - 1);          \
-    const int xs_ = max(1, min(FQ_XSHARE, 32 / cnt_)), xper_ = BT / xs_, xw_ = xper_ / NW;             \
+    const int xs_ = max(1, min(FQ_XSHARE, 32 / cnt_)), xper_ = BT / xs_, xw_ = xper_ / NW;     \
     xrow_ = ((pf_) % xs_) * xper_ + wave_u * xw_ + (lane < xw_ ? lane : 0);                    \
     xon_ = lane < xw_;                                                                         \
   }
+  // the sorted ids of the upper 128 slots of block pt_, two per lane: a block is a half tile when none holds a pair
+#define FQ_UPPER_IDS(pt_, u0_, u1_)                                \
+  {                                                                \
+    u0_ = a.sorted[(pt_) * BT + BT / 2 + lane];                    \
+    u1_ = a.sorted[(pt_) * BT + BT / 2 + kWave + lane];            \
+  }
+#define FQ_IS_HALF(u0_, u1_) (FQ_HALF && __ballot((u0_) < a.num_valid || (u1_) < a.num_valid) == 0)
 #define FQ_MAKE_SET(pt_, pf_, ex_, kb_, sh_, SIDOF, TSIDOF, xsrc_, wsrc_, xrs_, wrs_, tw_, tx_)                 \
   {                                                                                                          \
     const int64_t xrow0_ = a.top_k > 0 ? 0 : static_cast<int64_t>(pt_) * BT;                                 \
@@ -216,15 +234,31 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
     __builtin_amdgcn_raw_ptr_buffer_load_lds(wrs_, (lptr_t)(lds_raw + 2 * SLOT + wave_u * 256), 4, tw_, (tile_) * wstep, 0, 0);  \
     __builtin_amdgcn_raw_ptr_buffer_load_lds(xrs_, (lptr_t)(lds_raw + 2 * SLOT + wave_u * 256), 4, tx_, (tile_) * C::BKB, 0, 0); \
   }
-#define FQ_READ_W(buf_, j_, s_, sl_) fw[buf_][j_] = *reinterpret_cast<const u32x4*>(lds_raw + wadr[s_] + (sl_) * SLOT + FQ_WD(j_));
-#define FQ_READ_X(buf_, i_, s_, sl_) fx[buf_][i_] = *reinterpret_cast<const u32x4*>(lds_raw + xadr[s_] + (sl_) * SLOT + FQ_XD(i_));
-  // One K-step: 64 MFMAs from fragment buffer S.  FIRST: the accumulators start from zero.  RD: the fragments of
-  // K-step S ^ 1 of ring slot rsl_ are read into the other buffer.  LSET (0: none): the 16 loads of K tile ltile_
-  // of set LSET go into slot lsl_.  TCH: the touch (resources and offsets given) of K tile ttile_.
-#define FQ_KSTEP(S, FIRST, RD, rsl_, HAVE_LOAD, LSET, ltile_, lsl_, TCH, twrs_, txrs_, tw_, tx_, ttile_)   \
+#define FQ_READ_W(HALF, buf_, j_, s_, sl_) \
+  fw[buf_][j_] = *reinterpret_cast<const u32x4*>(lds_raw + wadr[s_] + ((HALF) ? wbaseH : wbaseF) + (sl_) * SLOT + FQ_WD(HALF, j_));
+#define FQ_READ_X(HALF, buf_, i_, s_, sl_) \
+  fx[buf_][i_] = *reinterpret_cast<const u32x4*>(lds_raw + xadr[s_] + ((HALF) ? 0 : xbaseF) + (sl_) * SLOT + FQ_XD(i_));
+  // read r of a K-step's fragment reads: whole tile X0 W0 X1 W1 ... (16), half tile X0 X1 W0 X2 X3 W1 ... (12)
+#define FQ_READ_NTH(HALF, r_, buf_, s_, sl_)                                                               \
   {                                                                                                        \
-    constexpr int RE = (S) == 0 ? RD0 : RD1;                                                               \
-    _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                                       \
+    if (HALF) {                                                                                            \
+      if ((r_) % 3 == 2) { FQ_READ_W(true, buf_, (r_) / 3, s_, sl_) }                                      \
+      else { FQ_READ_X(true, buf_, ((r_) / 3) * 2 + (r_) % 3, s_, sl_) }                                   \
+    } else {                                                                                               \
+      if ((r_) & 1) { FQ_READ_W(false, buf_, (r_) >> 1, s_, sl_) } else { FQ_READ_X(false, buf_, (r_) >> 1, s_, sl_) } \
+    }                                                                                                      \
+  }
+  // One K-step: the MFMAs of fragment buffer S (64, or 32 in a half tile: 4 weight x 8 token fragments).
+  // FIRST: the accumulators start from zero.  RD: the fragments of K-step S ^ 1 of ring slot rsl_ are read into
+  // the other buffer.  NLD_ (0: none): the first NLD_ loads of K tile ltile_ of set LSET go into slot lsl_.
+  // TCH: the touch (resources and offsets given) of K tile ttile_, behind the last load.
+#define FQ_KSTEP(HALF, S, FIRST, RD, rsl_, NLD_, LSET, ltile_, lsl_, TCH, twrs_, txrs_, tw_, tx_, ttile_)   \
+  {                                                                                                        \
+    constexpr int NMk = (HALF) ? NM / 2 : NM, NR = (HALF) ? NF + NF / 2 : 2 * NF;                          \
+    constexpr int RE = (HALF) ? 2 : ((S) == 0 ? RD0 : RD1);                                                \
+    constexpr int LP = (HALF) ? 1 : LD_POS, LE = (HALF) ? 2 : LD_EVERY;                                    \
+    static_assert(LP + (NL - 1) * LE < NMk && (NR - 1) * RE < NMk, "loads and reads fit the K-step");      \
+    _Pragma("unroll") for (int m = 0; m < NMk; ++m) {                                                      \
       const int j = m / NF, i = m % NF;                                                                    \
       if (FIRST) {                                                                                         \
         const f32x4 z_ = {0.f, 0.f, 0.f, 0.f};                                                             \
@@ -233,16 +267,15 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
         acc[j][i] = E::m16(&fw[S][j], &fx[S][i], acc[j][i]);                                               \
       }                                                                                                    \
       __builtin_amdgcn_sched_barrier(0);                                                                   \
-      if ((RD) && m % RE == 0 && m / RE < 2 * NF) {                                                        \
-        const int r = m / RE;                                                                              \
-        if (r & 1) { FQ_READ_W((S) ^ 1, r >> 1, (S) ^ 1, rsl_) } else { FQ_READ_X((S) ^ 1, r >> 1, (S) ^ 1, rsl_) } \
+      if ((RD) && m % RE == 0 && m / RE < NR) {                                                            \
+        FQ_READ_NTH(HALF, m / RE, (S) ^ 1, (S) ^ 1, rsl_)                                                  \
         __builtin_amdgcn_sched_barrier(0);                                                                 \
       }                                                                                                    \
-      if ((HAVE_LOAD) && m >= LD_POS && (m - LD_POS) % LD_EVERY == 0 && (m - LD_POS) / LD_EVERY < NL) {    \
-        FQ_ISSUE(LSET, ltile_, lsl_, (m - LD_POS) / LD_EVERY)                                              \
+      if ((NLD_) > 0 && m >= LP && (m - LP) % LE == 0 && (m - LP) / LE < (NLD_)) {                          \
+        FQ_ISSUE(LSET, ltile_, lsl_, (m - LP) / LE)                                                        \
         __builtin_amdgcn_sched_barrier(0);                                                                 \
       }                                                                                                    \
-      if ((TCH) && FQ_TOUCH && m == TOUCH_AT) {                                                            \
+      if ((TCH) && FQ_TOUCH && m == NMk - 1) {                                                             \
         FQ_TOUCH_ISSUE(twrs_, txrs_, tw_, tx_, ttile_)                                                     \
         __builtin_amdgcn_sched_barrier(0);                                                                 \
       }                                                                                                    \
@@ -262,19 +295,23 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
     __builtin_amdgcn_s_barrier();                                                        \
     __builtin_amdgcn_sched_barrier(0);                                                   \
   }
-  // A period: K tile t of the unit from ring slot par.  Touch of K tile t + ahead of this unit, or, past its end,
-  // of the next unit (NEXT; else the unit's last K tile once more).
-#define FQ_PERIOD_A(FIRST, ltile_, ttile_)                                                                         \
+  // A period: K tile t of the unit from ring slot par; its slot takes K tile ltile_ of the unit (a half tile loads
+  // the weight rows and the lower 128 token rows: 12 loads).  Touch of K tile ttile_ of the unit.
+#define FQ_PERIOD_A(HALF, FIRST, ltile_, ttile_)                                                                   \
   {                                                                                                                \
-    FQ_KSTEP(0, FIRST, true, par, false, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                                  \
+    FQ_KSTEP(HALF, 0, FIRST, true, par, 0, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                                \
     if (FIRST) FQ_SYNC0 else FQ_SYNC                                                                               \
-    FQ_KSTEP(1, false, true, par ^ 1, true, A, ltile_, par, true, wrsA, xrsA, twA, txA, ttile_)                    \
+    FQ_KSTEP(HALF, 1, false, true, par ^ 1, ((HALF) ? WI + XI / 2 : NL), A, ltile_, par, true, wrsA, xrsA, twA, txA, ttile_) \
     par ^= 1;                                                                                                      \
   }
-  // One work unit (an output tile, or a K slice of one): kn >= kQuadMinTiles K tiles.
-#define FQ_TILE(NEXT)                                                                                              \
+  // One work unit (an output tile, or a K slice of one): kn >= kQuadMinTiles K tiles.  The ring holds the unit's
+  // first two K tiles when it starts.  NEXT: the workgroup has another unit after this one, whose routing data is
+  // asked for at the start, turned into the address set B after two K tiles, and whose first two K tiles (all 16
+  // loads: its kind need not be this unit's) refill the ring during the last two K tiles of this one.
+#define FQ_TILE(NEXT, HALF)                                                                                        \
   {                                                                                                                \
     FQ_STAMP(0)                                                                                                    \
+    _Pragma("unroll") for (int r = 0; r < ((HALF) ? NF + NF / 2 : 2 * NF); ++r) FQ_READ_NTH(HALF, r, 0, 0, par)    \
     if (NEXT) {                                                                                                    \
       FQ_UNIT(unit + 1, n_pid_t, n_pid_f, n_expert, n_kb, n_kn, n_tu, shB)                                         \
       _Pragma("unroll") for (int q = 0; q < XI; ++q) {                                                             \
@@ -282,6 +319,7 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
         (void)c;                                                                                                   \
         n_sid[q] = a.sorted[n_pid_t * BT + rr];                                                                    \
       }                                                                                                            \
+      FQ_UPPER_IDS(n_pid_t, n_up0, n_up1)                                                                          \
       if (FQ_TOUCH) {                                                                                              \
         int wrow_, xrow_; bool xon_;                                                                               \
         FQ_TOUCH_ROWS(shB, n_pid_f, wrow_, xrow_, xon_)                                                            \
@@ -289,48 +327,60 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
         n_tsid = a.sorted[n_pid_t * BT + xrow_];                                                                   \
       }                                                                                                            \
     }                                                                                                              \
-    FQ_PERIOD_A(true, 2, kQuadTouchAhead)                                                                          \
-    FQ_PERIOD_A(false, 3, 1 + kQuadTouchAhead)                                                                     \
-    if (NEXT) FQ_MAKE_SET(n_pid_t, n_pid_f, n_expert, n_kb, shB, n_sid[q], n_tsid, xsrcB, wsrcB, xrsB, wrsB, twB, txB) \
+    FQ_PERIOD_A(HALF, true, 2, kQuadTouchAhead)                                                                    \
+    FQ_PERIOD_A(HALF, false, 3, 1 + kQuadTouchAhead)                                                               \
+    if (NEXT) {                                                                                                    \
+      FQ_MAKE_SET(n_pid_t, n_pid_f, n_expert, n_kb, shB, n_sid[q], n_tsid, xsrcB, wsrcB, xrsB, wrsB, twB, txB)     \
+      n_half = FQ_IS_HALF(n_up0, n_up1);                                                                           \
+    }                                                                                                              \
     __builtin_amdgcn_s_waitcnt(0xC07F); /* lgkmcnt(0): no scalar load pending inside the loop */                   \
-    for (int t = 2; t < kn - kQuadTouchAhead; ++t) FQ_PERIOD_A(false, t + 2, t + kQuadTouchAhead)                  \
+    for (int t = 2; t < kn - kQuadTouchAhead; ++t) FQ_PERIOD_A(HALF, false, t + 2, t + kQuadTouchAhead)            \
     if (NEXT) {                                                                                                    \
       /* the unit's last kQuadTouchAhead K tiles: touches go to the next unit's first K tiles */                   \
       int tb_ = 0;                                                                                                 \
       for (int t = kn - kQuadTouchAhead; t < kn - 2; ++t, ++tb_) {                                                 \
-        FQ_KSTEP(0, false, true, par, false, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                              \
+        FQ_KSTEP(HALF, 0, false, true, par, 0, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                            \
         FQ_SYNC                                                                                                    \
-        FQ_KSTEP(1, false, true, par ^ 1, true, A, t + 2, par, true, wrsB, xrsB, twB, txB, tb_)                    \
+        FQ_KSTEP(HALF, 1, false, true, par ^ 1, ((HALF) ? WI + XI / 2 : NL), A, t + 2, par, true, wrsB, xrsB, twB, txB, tb_) \
         par ^= 1;                                                                                                  \
       }                                                                                                            \
-      FQ_KSTEP(0, false, true, par, false, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                                \
+      FQ_KSTEP(HALF, 0, false, true, par, 0, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                              \
       FQ_SYNC                                                                                                      \
-      FQ_KSTEP(1, false, true, par ^ 1, true, B, 0, par, true, wrsB, xrsB, twB, txB, tb_)                          \
+      FQ_KSTEP(HALF, 1, false, true, par ^ 1, NL, B, 0, par, true, wrsB, xrsB, twB, txB, tb_)                      \
       par ^= 1;                                                                                                    \
-      FQ_KSTEP(0, false, true, par, false, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                                \
+      FQ_KSTEP(HALF, 0, false, true, par, 0, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                              \
       FQ_SYNC                                                                                                      \
-      FQ_KSTEP(1, false, true, par ^ 1, true, B, 1, par, true, wrsB, xrsB, twB, txB, tb_ + 1)                      \
+      FQ_KSTEP(HALF, 1, false, false, 0, NL, B, 1, par, true, wrsB, xrsB, twB, txB, tb_ + 1)                       \
       par ^= 1;                                                                                                    \
     } else {                                                                                                       \
-      for (int t = kn - kQuadTouchAhead; t < kn - 2; ++t) FQ_PERIOD_A(false, t + 2, kn - 1)                        \
-      FQ_KSTEP(0, false, true, par, false, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                                \
+      for (int t = kn - kQuadTouchAhead; t < kn - 2; ++t) FQ_PERIOD_A(HALF, false, t + 2, kn - 1)                  \
+      FQ_KSTEP(HALF, 0, false, true, par, 0, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                              \
       FQ_SYNC                                                                                                      \
-      FQ_KSTEP(1, false, true, par ^ 1, false, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                            \
+      FQ_KSTEP(HALF, 1, false, true, par ^ 1, 0, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                          \
       par ^= 1;                                                                                                    \
-      FQ_KSTEP(0, false, true, par, false, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                                \
+      FQ_KSTEP(HALF, 0, false, true, par, 0, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                              \
       FQ_SYNC0                                                                                                     \
-      FQ_KSTEP(1, false, false, 0, false, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                                 \
+      FQ_KSTEP(HALF, 1, false, false, 0, 0, A, 0, 0, false, wrsA, xrsA, twA, txA, 0)                               \
     }                                                                                                              \
     FQ_STAMP(1)                                                                                                    \
     /* the last MFMA's result is 16 cycles away: the fetches below are beyond the compiler's hazard checks */      \
-    asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");                                                              \
-    if (tu < 0) gemm_epilogue<T, C, EPI, true, true>(a, acc, pid_t, pid_f, expert, 0, wt, wf, frow, kgrp);         \
-    else tail_store<C, EPI, true>(a.tail_ws + static_cast<int64_t>(xcd * nper + tu) * (BT * BF), acc, wt, wf, frow, kgrp); \
+    asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");                                                               \
+    float* tws_ = a.tail_ws + static_cast<int64_t>(xcd * nper + (tu < 0 ? 0 : tu)) * (BT * BF);                    \
+    if (HALF) {                                                                                                    \
+      f32x4(&acch_)[NF / 2][NF] = reinterpret_cast<f32x4(&)[NF / 2][NF]>(acc);                                     \
+      if (tu < 0) gemm_epilogue<T, CH, EPI, true, true>(a, acch_, 2 * pid_t, pid_f, expert, 0, 0, wave_u, frow, kgrp); \
+      else tail_store<CH, EPI, true>(tws_, acch_, 0, wave_u, frow, kgrp);                                          \
+    } else {                                                                                                       \
+      if (tu < 0) gemm_epilogue<T, C, EPI, true, true>(a, acc, pid_t, pid_f, expert, 0, wt, wf, frow, kgrp);       \
+      else tail_store<C, EPI, true>(tws_, acc, wt, wf, frow, kgrp);                                                \
+    }                                                                                                              \
   }
 
   FQ_UNIT(0, pid_t, pid_f, expert, kb, kn, tu, shA)
   {
-    int tsid0 = 0;
+    int tsid0 = 0, up0, up1;
+    FQ_UPPER_IDS(pid_t, up0, up1)
+    half = FQ_IS_HALF(up0, up1);
     if (FQ_TOUCH) {
       int wrow_, xrow_; bool xon_;
       FQ_TOUCH_ROWS(shA, pid_f, wrow_, xrow_, xon_)
@@ -339,18 +389,13 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
     }
     FQ_MAKE_SET(pid_t, pid_f, expert, kb, shA, a.sorted[pid_t * BT + rr], tsid0, xsrcA, wsrcA, xrsA, wrsA, twA, txA)
   }
-  // fill: K tiles 0 and 1 into slots 0 and 1, then the fragments of the first K-step
+  // fill: K tiles 0 and 1 into slots 0 and 1
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int q = 0; q < NL; ++q) FQ_ISSUE(A, t, t, q)
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
   __builtin_amdgcn_s_barrier();
-#pragma unroll
-  for (int f = 0; f < NF; ++f) {
-    FQ_READ_W(0, f, 0, 0)
-    FQ_READ_X(0, f, 0, 0)
-  }
   int par = 0;
   int unit = 0;
 #ifdef FR_PROF  // cycle counts of wavefront 0 of every workgroup: K loops / epilogues and hand-over / total / K tiles
@@ -371,15 +416,15 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
 #define FQ_STAMP(k_)
 #endif
   for (; unit + 1 < n_units; ++unit) {
-    FQ_TILE(true)
+    if (half) FQ_TILE(true, true) else FQ_TILE(true, false)
     pid_t = n_pid_t; pid_f = n_pid_f; expert = n_expert; xrsA = xrsB; wrsA = wrsB;
-    kb = n_kb; kn = n_kn; tu = n_tu; twA = twB; txA = txB;
+    kb = n_kb; kn = n_kn; tu = n_tu; twA = twB; txA = txB; half = n_half;
 #pragma unroll
     for (int q = 0; q < XI; ++q) xsrcA[q] = xsrcB[q];
 #pragma unroll
     for (int q = 0; q < WI; ++q) wsrcA[q] = wsrcB[q];
   }
-  FQ_TILE(false)
+  if (half) FQ_TILE(false, true) else FQ_TILE(false, false)
   FQ_STAMP(2)
 #undef FQ_STAMP
 #undef FQ_TILE
@@ -387,11 +432,14 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
 #undef FQ_SYNC0
 #undef FQ_SYNC
 #undef FQ_KSTEP
+#undef FQ_READ_NTH
 #undef FQ_READ_X
 #undef FQ_READ_W
 #undef FQ_TOUCH_ISSUE
 #undef FQ_ISSUE
 #undef FQ_MAKE_SET
+#undef FQ_IS_HALF
+#undef FQ_UPPER_IDS
 #undef FQ_TOUCH_ROWS
 #undef FQ_XD
 #undef FQ_WD
