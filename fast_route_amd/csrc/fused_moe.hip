@@ -163,7 +163,11 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // (160 stays), 1536: 1148 / 1081, 1792: 1216 / 1102, 2048: 1395 / 1373, 2304: 1490 / 1626 (160 stays), 2560:
   // 1664 / 1647, 3072: 1973 / 1815, 5120: 3059 / 2911, 8192: 4804 / 4339.  Below 350 pairs per expert the smaller
   // tiles stream the weights faster (1024 tokens: 811 / 977 us).
-  if (two_byte && !g_tunables.no_quad && (block == 128 || block == 160) && H >= 4096 && F >= 1024 && E <= 1022 && avg >= 350) {
+  // With a short K (H = 2048, F = 1408, 64 experts: 32 and 22 K tiles per output tile) a tile's epilogue and hand-over
+  // weigh more and the gain is smaller and later: 160 / 256 rows 4096 tokens (384 pairs per expert) 568 / 587 us,
+  // 8192: 941 / 918, 16384: 1698 / 1637; taken from 700 pairs per expert on.
+  if (two_byte && !g_tunables.no_quad && (block == 128 || block == 160) && H >= 2048 && F >= 1024 && E <= 1022 &&
+      avg >= (H >= 4096 ? 350.0 : 700.0)) {
     const double other = expected(block) * block;
     const double quad = 0.5 * (expected(256) * 256 + expected(128) * 128);
     if (quad <= 1.08 * other) block = 256;

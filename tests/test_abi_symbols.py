@@ -59,8 +59,8 @@ def test_plan_table():
     H >= 4096, then 128 or - where the spread of the experts' loads around a multiple of 128 would cost
     every other expert one block more - 160; 2-byte operands take 256 rows (one wavefront per SIMD) from 350 pairs
     per expert on wherever their coarser blocks add less than 8 % of rows, 256 from 1200 pairs on otherwise; fp8 takes 160 rows only where
-    a sixth of the blocks go and 256 from 900 on; the fine-grained shape with H = 2048 has no 64-row range and never
-    takes 256 rows below 4096 pairs per expert)."""
+    a sixth of the blocks go and 256 from 900 on; the fine-grained shape with H = 2048 has no 64-row range and takes
+    256 rows from 700 pairs per expert on)."""
     from fast_route_amd import _native
     lib = _native.lib()
 
@@ -86,7 +86,7 @@ def test_plan_table():
     assert [mix(M, _native.FR_FP8_E4M3)[0] for M in (103, 104, 207, 208, 512, 768, 1024, 2048, 2560, 3600, 4096)] == \
         [32, 64, 64, 128, 160, 128, 160, 128, 160, 256, 256]
     fine = lambda M: plan(M, 2048, 1408, 64, 6)[0]
-    assert [fine(M) for M in (85, 86, 341, 342, 1246, 1247, 43690, 43691)] == [16, 32, 32, 128, 128, 160, 160, 256]
+    assert [fine(M) for M in (85, 86, 341, 342, 1246, 1247, 7466, 7467, 43691)] == [16, 32, 32, 128, 128, 160, 160, 256, 256]
     # the scratch for splitting the last round exists exactly for 128- and 256-row blocks with a long K
     p = _native.FrMoePlan()
     lib.fr_moe_get_plan(4096, 4096, 14336, 8, 2, _native.FR_BF16, p)
