@@ -166,11 +166,14 @@ extern "C" int fr_moe_get_plan(int64_t M, int64_t H, int64_t F, int E, int topk,
   // With a short K (H = 2048, F = 1408, 64 experts: 32 and 22 K tiles per output tile) a tile's epilogue and hand-over
   // weigh more and the gain is smaller and later: 160 / 256 rows 4096 tokens (384 pairs per expert) 568 / 587 us,
   // 8192: 941 / 918, 16384: 1698 / 1637; taken from 700 pairs per expert on.
-  if (two_byte && !g_tunables.no_quad && (block == 128 || block == 160) && H >= 2048 && F >= 1024 && E <= 1022 &&
-      avg >= (H >= 4096 ? 350.0 : 700.0)) {
+  // fp8 (32x32x64 MFMAs in that kernel; 16 K tiles are 2048 elements): 128 / 160 / 256 rows 2048 tokens 870 / - / 797 us,
+  // 2560: - / 1040 / 941, 4096: - / 1554 / 1383 (1511 on the eight-wavefront kernel), 16384: 5386 -> 4882.
+  if (!g_tunables.no_quad && (block == 128 || block == 160) && H >= 2048 && F >= 2048 / (two_byte ? 2 : 1) && E <= 1022 &&
+      avg >= (H >= 4096 ? (two_byte ? 350.0 : 300.0) : 700.0)) {
     const double other = expected(block) * block;
     const double quad = 0.5 * (expected(256) * 256 + expected(128) * 128);
-    if (quad <= 1.08 * other) block = 256;
+    // fp8 gains more per row (1280 tokens: 605 / 612 / 583 us with 128 / 160 / 256 rows, 2304: - / 882 / 870)
+    if (quad <= (two_byte ? 1.08 : 1.18) * other) block = 256;
   }
   if (g_tunables.block) block = g_tunables.block;
   // the fp8 160-row tile exists in the persistent form only (five K tiles per K slice at least, 1022 experts at most)

@@ -232,7 +232,17 @@ __device__ __forceinline__ f32x4 acc_fetch(const f32x4& v) {
 #else
 __device__ __forceinline__ f32x4 acc_fetch(const f32x4& v) { return v; }
 #endif
-__device__ __forceinline__ f32x16 acc_fetch(const f32x16& v) { return v; }
+__device__ __forceinline__ f32x16 acc_fetch(const f32x16& v) {
+  f32x16 o;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const f32x4 part = {v[g * 4 + 0], v[g * 4 + 1], v[g * 4 + 2], v[g * 4 + 3]};
+    const f32x4 got = acc_fetch(part);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[g * 4 + r] = got[r];
+  }
+  return o;
+}
 
 // AG: the accumulators live in the accumulation registers (one wavefront per SIMD) and are fetched tile by tile.
 template <typename T, typename C, int EPI, bool HOIST = true, bool AG = false, typename AccT>
@@ -317,12 +327,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
       constexpr int HJ = C::JF / 2;
       out_t* orow = static_cast<out_t*>(a.out) + static_cast<int64_t>(slot) * a.ldo;
 #pragma unroll
-      for (int j = 0; j < HJ; ++j)
+      for (int j = 0; j < HJ; ++j) {
+        const AccT ga = AG ? acc_fetch(acc[j][i]) : acc[j][i], ua = AG ? acc_fetch(acc[j + HJ][i]) : acc[j + HJ][i];
 #pragma unroll
         for (int g = 0; g < GROUPS; ++g) {
           const int f = pid_f * (BF / 2) + wf * (C::TF / 2) + j * C::TILE + g * 8 + kgrp * 4;
           out4 o;
-          const AccT ga = AG ? acc_fetch(acc[j][i]) : acc[j][i], ua = AG ? acc_fetch(acc[j + HJ][i]) : acc[j + HJ][i];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             float gv = ga[g * 4 + r], uv = ua[g * 4 + r];
@@ -338,16 +348,17 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
               if (f + r < a.N) orow[f + r] = o[r];
           if constexpr (kFence) __builtin_amdgcn_sched_barrier(0);
         }
+      }
     } else {
       if (sid < a.num_valid) {
         const float rw = routed[i] * xs;
 #pragma unroll
-        for (int j = 0; j < C::JF; ++j)
+        for (int j = 0; j < C::JF; ++j) {
+          const AccT ca = AG ? acc_fetch(acc[j][i]) : acc[j][i];
 #pragma unroll
           for (int g = 0; g < GROUPS; ++g) {
             const int f = pid_f * BF + wf * C::TF + j * C::TILE + g * 8 + kgrp * 4;
             float v[4];
-            const AccT ca = AG ? acc_fetch(acc[j][i]) : acc[j][i];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               v[r] = ca[g * 4 + r] * rw;
@@ -377,6 +388,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, AccT (&acc)[C::
             }
             if constexpr (kFence) __builtin_amdgcn_sched_barrier(0);
           }
+        }
       }
     }
   }

@@ -30,8 +30,13 @@
 
 namespace fr {
 
-typedef Cfg<256, 256, 128, 2, 2, 16, 1, 2, 0, 1> QuadCfg;
-typedef Cfg<128, 256, 128, 1, 4, 16, 1, 2, 0, 1> QuadHalfCfg;  // output geometry of a half tile: 128 rows, a quarter of the features per wavefront
+// 2-byte operands: 16x16x32 MFMAs (8 x 8 accumulator tiles of 4 registers per wavefront); fp8: 32x32x64 (4 x 4 tiles of
+// 16 registers).  Either way a K tile of 128 bytes per row is two K-steps, a K-step's fragments are 16 reads of 16
+// bytes per lane and 64 registers, and a wavefront issues 16 tile loads per K tile.
+template <typename T> struct QuadTile { static constexpr int kTile = sizeof(T) == 1 ? 32 : 16; };
+template <typename T> using QuadCfg = Cfg<256, 256, 128, 2, 2, QuadTile<T>::kTile, 1, 2, 0, 1>;
+// output geometry of a half tile: 128 rows, a quarter of the features per wavefront
+template <typename T> using QuadHalfCfg = Cfg<128, 256, 128, 1, 4, QuadTile<T>::kTile, 1, 2, 0, 1>;
 constexpr int kQuadMinTiles = 8;    // K tiles per work unit, at least (two peeled at each end, the touch distance)
 #ifndef FQ_AHEAD
 #define FQ_AHEAD 3
@@ -39,26 +44,8 @@ constexpr int kQuadMinTiles = 8;    // K tiles per work unit, at least (two peel
 constexpr int kQuadTouchAhead = FQ_AHEAD;  // K tiles between a touch and the tile loads of the same rows
 constexpr int kQuadSink = 1024;     // bytes of LDS the touches land in (256 per wavefront)
 
-#ifndef FQ_RD0
-#define FQ_RD0 3
-#endif
-#ifndef FQ_RD1
-#define FQ_RD1 4
-#endif
-#ifndef FQ_LD_POS
-#define FQ_LD_POS 2
-#endif
-#ifndef FQ_LD_EVERY
-#define FQ_LD_EVERY 4
-#endif
-#ifndef FQ_TOUCH_AT
-#define FQ_TOUCH_AT 63
-#endif
 #ifndef FQ_XSHARE
 #define FQ_XSHARE 4
-#endif
-#ifndef FQ_PRIO
-#define FQ_PRIO 0
 #endif
 #ifndef FQ_HALF
 #define FQ_HALF 1
@@ -70,19 +57,24 @@ constexpr int kQuadSink = 1024;     // bytes of LDS the touches land in (256 per
 template <typename T, int EPI>
 __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a FR_PROF_PARAM) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  typedef QuadCfg C;
-  typedef QuadHalfCfg CH;
+  typedef QuadCfg<T> C;
+  typedef QuadHalfCfg<T> CH;
   typedef Elem<T> E;
   typedef __attribute__((address_space(3))) void* lptr_t;
-  static_assert(sizeof(T) == 2, "2-byte operands");
-  constexpr int BT = C::BT, BF = C::BF, CPR = C::CPR, BK = C::BKB / 2, EPC = 8;
-  constexpr int NF = 8;                       // fragments per operand and K-step
-  constexpr int NM = NF * NF;                 // MFMAs per K-step
+  typedef typename std::conditional<C::TILE == 32, f32x16, f32x4>::type acc_t;
+  constexpr int ES = static_cast<int>(sizeof(T));
+  constexpr int BT = C::BT, BF = C::BF, CPR = C::CPR, BK = C::BKB / ES, EPC = 16 / ES, FC = E::FC;
+  constexpr int TILE = C::TILE, KG = C::KGROUPS;
+  constexpr int NF = 128 / TILE;              // fragments per operand and K-step (8, fp8: 4)
+  constexpr int NM = NF * NF;                 // MFMAs per K-step (64 of 16 cycles, fp8: 16 of 64 cycles)
   constexpr int NW = 4, XI = 8, WI = 8, NL = XI + WI;  // tile loads per wavefront and K tile
   constexpr int XBYTES = C::XCH * 16, WBYTES = C::WCH * 16, SLOT = XBYTES + WBYTES;  // a ring slot: X rows, then W rows
-  constexpr int RD0 = FQ_RD0, RD1 = FQ_RD1;   // one fragment read after every n-th MFMA of the first / second K-step
-  constexpr int LD_POS = FQ_LD_POS, LD_EVERY = FQ_LD_EVERY;  // tile load q after MFMA LD_POS + q * LD_EVERY of the second K-step
-  static_assert(C::IT == NF && C::JF == NF && C::XIW == XI && C::WIW == WI && C::KGROUPS == 4 && CPR == 8, "128 x 128 per wavefront");
+  // Whole tile, 2-byte operands: one fragment read after every 3rd / 4th MFMA of the first / second K-step, tile
+  // load q after MFMA 2 + 4 q of the second.  fp8 has a quarter of the MFMAs, four times as long: two fragment reads
+  // after each of the first eight, one tile load after every one of the second K-step.
+  constexpr int RD0 = FC == 1 ? 3 : 1, RD1 = FC == 1 ? 4 : 1, RPS = FC;
+  constexpr int LD_POS = FC == 1 ? 2 : 0, LD_EVERY = FC == 1 ? 4 : 1;
+  static_assert(C::IT == NF && C::JF == NF && C::XIW == XI && C::WIW == WI && CPR == 8 && CPR / (KG * FC) == 2, "128 x 128 per wavefront, two K-steps per K tile");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
 
@@ -139,22 +131,21 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
   // rows acc_tile_col<CH>(w, .) - a quarter of the features each, so that the four MFMA pipes share what is left.
   // All of a lane's fragment rows lie multiples of 16 apart (one swizzle key), and the two forms differ by
   // wavefront-uniform distances.
-  const int frow = lane & 15, kgrp = lane >> 4;
+  const int frow = lane % TILE, kgrp = lane / TILE;
   const int key0 = swizzle<CPR>(frow, 0);
-  int xadr[2], wadr[2];  // byte addresses in slot 0 of the fragments of row frow of the X tile / the W tile
+  int xadr[2][FC];  // byte addresses in slot 0 of the chunks of row frow of the X tile (the W tile: XBYTES further)
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    xadr[s] = (frow * CPR + ((s * 4 + kgrp) ^ key0)) * 16;
-    wadr[s] = XBYTES + xadr[s];
-  }
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int c = 0; c < FC; ++c) xadr[s][c] = (frow * CPR + (((s * KG + kgrp) * FC + c) ^ key0)) * 16;
   const int xbaseF = wt * C::TT * CPR * 16, wbaseF = acc_tile_col<C, EPI>(wf, 0) * CPR * 16;
   const int wbaseH = acc_tile_col<CH, EPI>(wave_u, 0) * CPR * 16;
-#define FQ_XD(i_) ((i_) * 16 * CPR * 16)
+#define FQ_XD(i_) ((i_) * TILE * CPR * 16)
 #define FQ_WD(HALF, j_) ((HALF) ? (acc_tile_col<CH, EPI>(0, (j_)) - acc_tile_col<CH, EPI>(0, 0)) * CPR * 16 \
                                : (acc_tile_col<C, EPI>(0, (j_)) - acc_tile_col<C, EPI>(0, 0)) * CPR * 16)
 
-  f32x4 acc[NF][NF];
-  u32x4 fw[2][NF], fx[2][NF];
+  acc_t acc[NF][NF];
+  u32x4 fw[2][NF][FC], fx[2][NF][FC];
 
   // ---- address sets: A = unit being multiplied, B = the workgroup's next unit ---------------------
   int pid_t, pid_f, expert, kb, kn, tu;
@@ -196,22 +187,22 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
       int64_t row_ = rr;                                                                                     \
       const int sid_ = SIDOF;                                                                                \
       if (a.top_k > 0) row_ = sid_ < a.num_valid ? sid_ / a.top_k : 0;                                       \
-      xsrc_[q] = static_cast<unsigned>((row_ * a.ldx + kfirst_ + c * EPC) * 2);                              \
+      xsrc_[q] = static_cast<unsigned>((row_ * a.ldx + kfirst_ + c * EPC) * ES);                              \
       if (a.x_span && sid_ >= a.num_valid) xsrc_[q] = kSkipOffset;                                           \
     }                                                                                                        \
     _Pragma("unroll") for (int q = 0; q < WI; ++q) {                                                         \
       FQ_SLOT_ROW(q, rr, c)                                                                                  \
-      wsrc_[q] = static_cast<unsigned>(w_byte_offset(a.w_tiled, a.ldw, a.K, w_src_row(pf_, rr), (kfirst_ + c * EPC) * 2, 2)); \
+      wsrc_[q] = static_cast<unsigned>(w_byte_offset(a.w_tiled, a.ldw, a.K, w_src_row(pf_, rr), (kfirst_ + c * EPC) * ES, ES)); \
     }                                                                                                        \
     if (FQ_TOUCH) {                                                                                          \
       int wrow_, xrow_; bool xon_;                                                                           \
       FQ_TOUCH_ROWS(sh_, pf_, wrow_, xrow_, xon_)                                                            \
       (void)xrow_;                                                                                           \
-      tw_ = static_cast<unsigned>(w_byte_offset(a.w_tiled, a.ldw, a.K, w_src_row(pf_, wrow_), kfirst_ * 2, 2)); \
+      tw_ = static_cast<unsigned>(w_byte_offset(a.w_tiled, a.ldw, a.K, w_src_row(pf_, wrow_), kfirst_ * ES, ES)); \
       int64_t trow_ = xrow_;                                                                                 \
       const int tsid_ = TSIDOF;                                                                              \
       if (a.top_k > 0) trow_ = tsid_ < a.num_valid ? tsid_ / a.top_k : 0;                                    \
-      tx_ = static_cast<unsigned>((trow_ * a.ldx + kfirst_) * 2);                                            \
+      tx_ = static_cast<unsigned>((trow_ * a.ldx + kfirst_) * ES);                                            \
       if (a.x_span && (tsid_ >= a.num_valid || !xon_)) tx_ = kSkipOffset;                                    \
     }                                                                                                        \
   }
@@ -234,46 +225,59 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
     __builtin_amdgcn_raw_ptr_buffer_load_lds(wrs_, (lptr_t)(lds_raw + 2 * SLOT + wave_u * 256), 4, tw_, (tile_) * wstep, 0, 0);  \
     __builtin_amdgcn_raw_ptr_buffer_load_lds(xrs_, (lptr_t)(lds_raw + 2 * SLOT + wave_u * 256), 4, tx_, (tile_) * C::BKB, 0, 0); \
   }
-#define FQ_READ_W(HALF, buf_, j_, s_, sl_) \
-  fw[buf_][j_] = *reinterpret_cast<const u32x4*>(lds_raw + wadr[s_] + ((HALF) ? wbaseH : wbaseF) + (sl_) * SLOT + FQ_WD(HALF, j_));
-#define FQ_READ_X(HALF, buf_, i_, s_, sl_) \
-  fx[buf_][i_] = *reinterpret_cast<const u32x4*>(lds_raw + xadr[s_] + ((HALF) ? 0 : xbaseF) + (sl_) * SLOT + FQ_XD(i_));
-  // read r of a K-step's fragment reads: whole tile X0 W0 X1 W1 ... (16), half tile X0 X1 W0 X2 X3 W1 ... (12)
+#define FQ_READ_W(HALF, buf_, j_, c_, s_, sl_)                                                             \
+  fw[buf_][j_][c_] = *reinterpret_cast<const u32x4*>(lds_raw + XBYTES + xadr[s_][c_] + ((HALF) ? wbaseH : wbaseF) + \
+                                                     (sl_) * SLOT + FQ_WD(HALF, j_));
+#define FQ_READ_X(HALF, buf_, i_, c_, s_, sl_) \
+  fx[buf_][i_][c_] = *reinterpret_cast<const u32x4*>(lds_raw + xadr[s_][c_] + ((HALF) ? 0 : xbaseF) + (sl_) * SLOT + FQ_XD(i_));
+  // read r of a K-step's fragment reads (FC chunks per fragment): whole tile X0 W0 X1 W1 ..., half tile X0 X1 W0
+  // X2 X3 W1 ... (twice as many token as weight fragments)
 #define FQ_READ_NTH(HALF, r_, buf_, s_, sl_)                                                               \
   {                                                                                                        \
+    const int f_ = (r_) / FC, c_ = (r_) % FC;                                                          \
     if (HALF) {                                                                                            \
-      if ((r_) % 3 == 2) { FQ_READ_W(true, buf_, (r_) / 3, s_, sl_) }                                      \
-      else { FQ_READ_X(true, buf_, ((r_) / 3) * 2 + (r_) % 3, s_, sl_) }                                   \
+      if (f_ % 3 == 2) { FQ_READ_W(true, buf_, f_ / 3, c_, s_, sl_) }                                      \
+      else { FQ_READ_X(true, buf_, (f_ / 3) * 2 + f_ % 3, c_, s_, sl_) }                                   \
     } else {                                                                                               \
-      if ((r_) & 1) { FQ_READ_W(false, buf_, (r_) >> 1, s_, sl_) } else { FQ_READ_X(false, buf_, (r_) >> 1, s_, sl_) } \
+      if (f_ & 1) { FQ_READ_W(false, buf_, f_ >> 1, c_, s_, sl_) } else { FQ_READ_X(false, buf_, f_ >> 1, c_, s_, sl_) } \
     }                                                                                                      \
   }
-  // One K-step: the MFMAs of fragment buffer S (64, or 32 in a half tile: 4 weight x 8 token fragments).
+  // One K-step: the MFMAs of fragment buffer S (a half tile: half as many, its weight fragments are half).
   // FIRST: the accumulators start from zero.  RD: the fragments of K-step S ^ 1 of ring slot rsl_ are read into
   // the other buffer.  NLD_ (0: none): the first NLD_ loads of K tile ltile_ of set LSET go into slot lsl_.
   // TCH: the touch (resources and offsets given) of K tile ttile_, behind the last load.
 #define FQ_KSTEP(HALF, S, FIRST, RD, rsl_, NLD_, LSET, ltile_, lsl_, TCH, twrs_, txrs_, tw_, tx_, ttile_)   \
   {                                                                                                        \
-    constexpr int NMk = (HALF) ? NM / 2 : NM, NR = (HALF) ? NF + NF / 2 : 2 * NF;                          \
-    constexpr int RE = (HALF) ? 2 : ((S) == 0 ? RD0 : RD1);                                                \
-    constexpr int LP = (HALF) ? 1 : LD_POS, LE = (HALF) ? 2 : LD_EVERY;                                    \
-    static_assert(LP + (NL - 1) * LE < NMk && (NR - 1) * RE < NMk, "loads and reads fit the K-step");      \
+    constexpr int NMk = (HALF) ? NM / 2 : NM, NR = ((HALF) ? NF + NF / 2 : 2 * NF) * FC;                   \
+    constexpr int RE = (HALF) ? (FC == 1 ? 2 : 1) : ((S) == 0 ? RD0 : RD1);                                \
+    constexpr int LP = (HALF) ? (FC == 1 ? 1 : 0) : LD_POS, LE = (HALF) ? (FC == 1 ? 2 : 1) : LD_EVERY;    \
+    constexpr int LPS = ((HALF) && FC == 2) ? 2 : 1;  /* loads per MFMA slot */                            \
+    static_assert(LP + ((NL + LPS - 1) / LPS - 1) * LE < NMk && ((NR + RPS - 1) / RPS - 1) * RE < NMk,     \
+                  "loads and reads fit the K-step");                                                       \
     _Pragma("unroll") for (int m = 0; m < NMk; ++m) {                                                      \
       const int j = m / NF, i = m % NF;                                                                    \
       if (FIRST) {                                                                                         \
-        const f32x4 z_ = {0.f, 0.f, 0.f, 0.f};                                                             \
-        acc[j][i] = E::m16(&fw[S][j], &fx[S][i], z_);                                                      \
+        const acc_t z_ = {};                                                                               \
+        if constexpr (TILE == 32) acc[j][i] = E::m32(fw[S][j], fx[S][i], z_);                              \
+        else acc[j][i] = E::m16(fw[S][j], fx[S][i], z_);                                                   \
       } else {                                                                                             \
-        acc[j][i] = E::m16(&fw[S][j], &fx[S][i], acc[j][i]);                                               \
+        if constexpr (TILE == 32) acc[j][i] = E::m32(fw[S][j], fx[S][i], acc[j][i]);                       \
+        else acc[j][i] = E::m16(fw[S][j], fx[S][i], acc[j][i]);                                            \
       }                                                                                                    \
       __builtin_amdgcn_sched_barrier(0);                                                                   \
-      if ((RD) && m % RE == 0 && m / RE < NR) {                                                            \
-        FQ_READ_NTH(HALF, m / RE, (S) ^ 1, (S) ^ 1, rsl_)                                                  \
-        __builtin_amdgcn_sched_barrier(0);                                                                 \
+      if ((RD) && m % RE == 0) {                                                                           \
+        _Pragma("unroll") for (int rr = 0; rr < RPS; ++rr)                                                 \
+          if ((m / RE) * RPS + rr < NR) {                                                                  \
+            FQ_READ_NTH(HALF, (m / RE) * RPS + rr, (S) ^ 1, (S) ^ 1, rsl_)                                 \
+            __builtin_amdgcn_sched_barrier(0);                                                             \
+          }                                                                                                \
       }                                                                                                    \
-      if ((NLD_) > 0 && m >= LP && (m - LP) % LE == 0 && (m - LP) / LE < (NLD_)) {                          \
-        FQ_ISSUE(LSET, ltile_, lsl_, (m - LP) / LE)                                                        \
-        __builtin_amdgcn_sched_barrier(0);                                                                 \
+      if ((NLD_) > 0 && m >= LP && (m - LP) % LE == 0) {                                                   \
+        _Pragma("unroll") for (int ll = 0; ll < LPS; ++ll)                                                 \
+          if (((m - LP) / LE) * LPS + ll < (NLD_)) {                                                       \
+            FQ_ISSUE(LSET, ltile_, lsl_, ((m - LP) / LE) * LPS + ll)                                       \
+            __builtin_amdgcn_sched_barrier(0);                                                             \
+          }                                                                                                \
       }                                                                                                    \
       if ((TCH) && FQ_TOUCH && m == NMk - 1) {                                                             \
         FQ_TOUCH_ISSUE(twrs_, txrs_, tw_, tx_, ttile_)                                                     \
@@ -311,7 +315,7 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
 #define FQ_TILE(NEXT, HALF)                                                                                        \
   {                                                                                                                \
     FQ_STAMP(0)                                                                                                    \
-    _Pragma("unroll") for (int r = 0; r < ((HALF) ? NF + NF / 2 : 2 * NF); ++r) FQ_READ_NTH(HALF, r, 0, 0, par)    \
+    _Pragma("unroll") for (int r = 0; r < ((HALF) ? NF + NF / 2 : 2 * NF) * FC; ++r) FQ_READ_NTH(HALF, r, 0, 0, par) \
     if (NEXT) {                                                                                                    \
       FQ_UNIT(unit + 1, n_pid_t, n_pid_f, n_expert, n_kb, n_kn, n_tu, shB)                                         \
       _Pragma("unroll") for (int q = 0; q < XI; ++q) {                                                             \
@@ -367,7 +371,7 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
     asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");                                                               \
     float* tws_ = a.tail_ws + static_cast<int64_t>(xcd * nper + (tu < 0 ? 0 : tu)) * (BT * BF);                    \
     if (HALF) {                                                                                                    \
-      f32x4(&acch_)[NF / 2][NF] = reinterpret_cast<f32x4(&)[NF / 2][NF]>(acc);                                     \
+      acc_t(&acch_)[NF / 2][NF] = reinterpret_cast<acc_t(&)[NF / 2][NF]>(acc);                                     \
       if (tu < 0) gemm_epilogue<T, CH, EPI, true, true>(a, acch_, 2 * pid_t, pid_f, expert, 0, 0, wave_u, frow, kgrp); \
       else tail_store<CH, EPI, true>(tws_, acch_, 0, wave_u, frow, kgrp);                                          \
     } else {                                                                                                       \
@@ -451,7 +455,7 @@ __global__ __launch_bounds__(256, 1) void moe_gemm_quad_kernel(const GemmArgs a 
 // Workgroups resident at once on the current device: one per CU (a multiple of 8, one share per XCD).
 template <typename T, int EPI>
 int quad_grid(int* grid_out) {
-  typedef QuadCfg C;
+  typedef QuadCfg<T> C;
   constexpr int kMaxDevices = 64;
   constexpr int kLds = C::LDS_BYTES + kQuadSink;
   static int cached[kMaxDevices] = {};  // per device; a race between threads writes the same value twice
@@ -480,9 +484,9 @@ int quad_grid(int* grid_out) {
 // launch_gemm_persistent).
 template <typename T, int EPI>
 int launch_gemm_quad(const GemmArgs& a_in, int splits, hipStream_t st) {
-  typedef QuadCfg C;
+  typedef QuadCfg<T> C;
   GemmArgs a = a_in;
-  constexpr int BK = C::BKB / 2;
+  constexpr int ES = static_cast<int>(sizeof(T)), BK = C::BKB / ES;
   if (a.setup_only) {
     int resident = 0;
     return quad_grid<T, EPI>(&resident);
@@ -492,12 +496,12 @@ int launch_gemm_quad(const GemmArgs& a_in, int splits, hipStream_t st) {
   const int64_t x_rows = a.top_k > 0 ? a.num_valid / a.top_k : C::BT;
   const int64_t w_rows = EPI == EPI_SILU ? 2 * static_cast<int64_t>(a.N) : a.N;
   const int64_t lim = int64_t(1) << 32;
-  if (x_rows * a.ldx * 2 >= lim || w_rows * a.ldw * 2 >= lim)
+  if (x_rows * a.ldx * ES >= lim || w_rows * a.ldw * ES >= lim)
     return fail(FR_E_SHAPE, "token rows (%lld x %lld) or one expert's weights (%lld x %lld) span 4 GiB or more",
                 (long long)x_rows, (long long)a.ldx, (long long)w_rows, (long long)a.ldw);
   a.group_t = tunables().group_m ? tunables().group_m : kChunkBlocks;
   if (tunables().no_tail_split) a.tail_ws = nullptr;
-  a.x_span = x_rows * a.ldx * 2 < (int64_t(1) << 31) ? static_cast<unsigned>(x_rows * a.ldx * 2) : 0u;
+  a.x_span = x_rows * a.ldx * ES < (int64_t(1) << 31) ? static_cast<unsigned>(x_rows * a.ldx * ES) : 0u;
   int resident = 0;
   const int rc = quad_grid<T, EPI>(&resident);
   if (rc != FR_OK) return rc;

@@ -86,15 +86,15 @@ int dispatch_block(GemmArgs a, int block, int splits, int64_t sorted_len, hipStr
       // faster for the down projection, but 6 % slower for the gate/up GEMM (short K, register-starved
       // epilogue: the hand-off K tiles spill; without the hand-off it is within 1 % of the plain kernel),
       // which keeps the plain kernel.
+      // one wavefront per SIMD, 128 x 128 outputs each (see moe_gemm_quad.h), where its K loop is long enough
+      if (!tunables().no_quad) {
+        const int rc = launch_gemm_quad<T, EPI>(a, splits, st);
+        if (rc != 1) return rc;
+      }
       if constexpr (sizeof(T) == 1 && EPI == EPI_SILU) return launch_gemm<T, typename TL::T256G, EPI>(a, splits, st);
       else {
         // 2-byte operands, long K: the 16x16x32 MFMA form (see Tiles::T256S)
         if constexpr (sizeof(T) == 2) {
-          // one wavefront per SIMD, 128 x 128 outputs each (see moe_gemm_quad.h), where its K loop is long enough
-          if (!tunables().no_quad) {
-            const int rc = launch_gemm_quad<T, EPI>(a, splits, st);
-            if (rc != 1) return rc;
-          }
           if (a.K >= kSmallMfmaMinK) return launch_gemm_persistent<T, typename TL::T256S, EPI>(a, splits, st);
         }
         return launch_gemm_persistent<T, typename TL::T256, EPI>(a, splits, st);
@@ -151,8 +151,8 @@ int prepare_tiles() {
   int rc = launch_gemm_persistent<T, typename TL::T256, EPI>(a, 1, nullptr);
   if constexpr (sizeof(T) == 2) {
     if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T256S, EPI>(a, 1, nullptr);
-    if (rc == FR_OK) rc = launch_gemm_quad<T, EPI>(a, 1, nullptr);
   }
+  if (rc == FR_OK) rc = launch_gemm_quad<T, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T128P, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm_persistent<T, typename TL::T160P, EPI>(a, 1, nullptr);
   if (rc == FR_OK) rc = launch_gemm<T, typename TL::T128, EPI>(a, 1, nullptr);

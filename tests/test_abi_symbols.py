@@ -83,8 +83,8 @@ def test_plan_table():
     assert mix(1) == (16, 4) and mix(2) == (16, 2) and mix(3) == (16, 4) and mix(4) == (16, 4) and mix(16) == (16, 1)
     assert mix(128) == (64, 2)
     assert mix(4096)[1] == 1 and plan(16384, 4096, 14336, 8, 2)[0] == 256
-    assert [mix(M, _native.FR_FP8_E4M3)[0] for M in (103, 104, 207, 208, 512, 768, 1024, 2048, 2560, 3600, 4096)] == \
-        [32, 64, 64, 128, 160, 128, 160, 128, 160, 256, 256]
+    assert [mix(M, _native.FR_FP8_E4M3)[0] for M in (103, 104, 207, 208, 512, 768, 1024, 1200, 1280, 2048, 2304, 2560, 4096)] == \
+        [32, 64, 64, 128, 160, 128, 160, 160, 256, 256, 256, 256, 256]
     fine = lambda M: plan(M, 2048, 1408, 64, 6)[0]
     assert [fine(M) for M in (85, 86, 341, 342, 1246, 1247, 7466, 7467, 43691)] == [16, 32, 32, 128, 128, 160, 160, 256, 256]
     # the scratch for splitting the last round exists exactly for 128- and 256-row blocks with a long K
