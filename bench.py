@@ -263,10 +263,13 @@ def kernel_roofline(shape, rec, fp8=False):
     byts = rec["active_experts"] * 2 * F * H * eb + M * H * eb + M * topk * F * 2
     peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
     # which kernel the library picks for the gate/up GEMM: weight rows against token rows for up to 4
-    # tokens of 2-byte operands with H = 4096, 5120, 6144, 7168 or 8192, the persistent tile kernel for 128- and 160-row
-    # blocks and for 256-row blocks of 2-byte operands, the plain tile kernel otherwise
+    # tokens of 2-byte operands with H = 4096, 5120, 6144, 7168 or 8192, the one-wavefront-per-SIMD kernel for 256-row
+    # blocks with a K of 16 K tiles or more, the persistent tile kernel for 64-, 128- and 160-row blocks (and 256-row
+    # blocks of 2-byte operands with a short K), the plain tile kernel otherwise
     if not fp8 and M <= 4 and H >= 4096 and H % 512 == 0 and any(H // 512 % c == 0 for c in (5, 6, 7, 8)) and M * H * 2 <= 65536:
         name = "gateup_rows_kernel"
+    elif rec["block"] == 256 and H >= (2048 if fp8 else 1024):  # 16 K tiles of 128 bytes per row or more
+        name = "moe_gemm_quad_kernel<EPI_SILU>"
     elif rec["block"] in (64, 128, 160) or (rec["block"] == 256 and not fp8):
         name = "moe_gemm_persistent_kernel<EPI_SILU>"
     else:
@@ -290,7 +293,7 @@ def tunables_now(N):
     return {name: int(getattr(t, name)) for name, _ in t._fields_}
 
 
-GEMM_KERNEL_SOURCES = ("moe_gemm_kernel.h", "moe_gemm_persistent.h", "moe_gemm_tiles.h", "moe_gemv.h", "moe_gemm.hip")
+GEMM_KERNEL_SOURCES = ("moe_gemm_kernel.h", "moe_gemm_persistent.h", "moe_gemm_quad.h", "moe_gemm_tiles.h", "moe_gemv.h", "moe_gemm.hip")
 
 
 def kernel_sources_sha():

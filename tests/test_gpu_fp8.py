@@ -146,6 +146,38 @@ def test_fp8_down_projection_tail_split(native, rows256):
     assert (o - ref).abs().max() <= 2.0 ** -5 * ref.abs().max()
 
 
+def test_fp8_one_wavefront_per_simd_tile_equals_the_eight_wavefront_tile(native):
+    """fp8 on 256-row blocks with 16 K tiles (2048 elements) or more runs on four wavefronts of 128 x 128 outputs
+    (moe_gemm_quad_kernel, 32x32x64 MFMAs); the no_quad knob sends the call to the eight-wavefront kernels.  Same
+    MFMA shape and K order: equal bit for bit, and within the fp8 bounds of the oracle.  Sixteen experts with a mix
+    of full, under-half and over-half blocks (half tiles), 2304 and 2560 elements of K (18 and 20 K tiles); top-2
+    routing by logits."""
+    import fast_route_amd as fr
+    from fast_route_amd import fused_moe_fp8, prepare_weights_fp8
+    _say("fp8 quad tile vs eight-wavefront tile")
+    H, Fd, E, k, M = 2304, 2560, 16, 2, 2600
+    g = torch.Generator().manual_seed(93)
+    x = torch.randn(M, H, generator=g).bfloat16()
+    w1 = (torch.randn(E, 2 * Fd, H, generator=g) * 0.02).bfloat16()
+    w2 = (torch.randn(E, H, Fd, generator=g) * 0.02).bfloat16()
+    logits = torch.randn(M, E, generator=g) + torch.linspace(2.0, -2.0, E)  # skewed loads: 1 .. 3 blocks per expert
+    w1q, w1s, w2q, w2s = prepare_weights_fp8(w1.cuda(), w2.cuda())
+    try:
+        with fr.tunables(block=256):
+            quad = fused_moe_fp8(x.cuda(), w1q, w1s, w2q, w2s, logits.cuda(), k, True)
+        with fr.tunables(block=256, no_quad=True):
+            eight = fused_moe_fp8(x.cuda(), w1q, w1s, w2q, w2s, logits.cuda(), k, True)
+        torch.cuda.synchronize()
+    finally:
+        fr.reset_tunables()
+    assert torch.equal(quad, eight), "the two 256-row fp8 kernels differ"
+    ref, _ = oracle.fused_moe_fp8(x, w1, w2, logits, k, True)
+    o = quad.float().cpu()
+    assert torch.isfinite(o).all()
+    assert (o - ref).norm() / ref.norm() <= 1e-2
+    assert (o - ref).abs().max() <= 2.0 ** -5 * ref.abs().max()
+
+
 def test_fp8_random_shapes_against_oracle(native):
     """Sixteen seeded random fp8 layer shapes against the oracle (same tolerance as above)."""
     from fast_route_amd import fused_moe_fp8, prepare_weights_fp8

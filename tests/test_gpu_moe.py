@@ -695,6 +695,17 @@ def test_one_wavefront_per_simd_tile_equals_the_eight_wavefront_tile(native, dty
         torch.cuda.synchronize()
         assert torch.equal(a, b), "the two 256-row kernels differ (layer with gating)"
         _assert_close(a, oracle.fused_moe(x2, w1b, w2b, logits, 2, True), dtype, "quad tile, layer")
+        # widths that are no multiples of 256: 18 and 22 K tiles, the down projection's last feature tile half wide;
+        # three experts, one of them without a token
+        x3, logits3, w1c, w2c = _inputs(900, 1152, 1408, 3, 79, dtype)
+        logits3[:, 1] = -30.0
+        with fr.tunables(block=256):
+            c = fused_moe(x3.cuda(), w1c.cuda(), w2c.cuda(), logits3.cuda(), 2, True)
+        with fr.tunables(block=256, no_quad=True):
+            d = fused_moe(x3.cuda(), w1c.cuda(), w2c.cuda(), logits3.cuda(), 2, True)
+        torch.cuda.synchronize()
+        assert torch.equal(c, d), "the two 256-row kernels differ (odd widths)"
+        _assert_close(c, oracle.fused_moe(x3, w1c, w2c, logits3, 2, True), dtype, "quad tile, odd widths")
     finally:
         fr.reset_tunables()
 
