@@ -1,5 +1,5 @@
 // Persistent grouped GEMM with ONE wavefront per SIMD: 256 sorted slots x 256 features per workgroup, four
-// wavefronts of 128 x 128 each, 16x16x32 MFMAs (2-byte operands).
+// wavefronts of 128 x 128 each, 16x16x32 MFMAs (2-byte operands) or 32x32x64 MFMAs (fp8).
 //
 // Why.  In the eight-wavefront tiles a wavefront owns 128 x 64 outputs and reads twelve operand fragments from
 // LDS for thirty-two MFMAs; with 128 x 128 per wavefront it reads sixteen for sixty-four, a third less LDS traffic
@@ -23,8 +23,17 @@
 // rows), and each of them asks for its share of the rows of a K tile several K tiles ahead - one dword per
 // 128-byte row piece, into a sink in LDS - so that the tile loads proper find their lines in L2.
 //
+// Half tiles.  A block whose upper 128 slots are all padding (the last block of every other expert) is multiplied
+// as 128 rows x 256 features with the FEATURES split four ways over the wavefronts (128 x 64 each): half the MFMAs
+// per K-step, 12 loads per K tile.  Both forms of the K loop exist for every place in the persistent walk; the kind
+// of the next unit is known a tile ahead, and the hand-over always loads a whole tile's first two K tiles, so any
+// kind may follow any other.
+//
 // Same tile walk, tail split, LDS swizzle, epilogues and fix-up kernel as moe_gemm_persistent_kernel; the result
-// is bit-identical to its 16x16x32 form (same MFMA shape, same K order per accumulator).
+// is bit-identical to the eight-wavefront kernels on the same MFMA shape (same K order per accumulator).
+//
+// Measurement switches (compile time, -D): FQ_TOUCH=0 no L2 touch, FQ_HALF=0 no half tiles, FQ_AHEAD=n touch
+// distance in K tiles, FQ_XSHARE=n ways the token rows' touch is shared; results stay correct with all of them.
 #pragma once
 #include "moe_gemm_persistent.h"
 
