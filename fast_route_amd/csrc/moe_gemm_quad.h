@@ -517,9 +517,12 @@ int launch_gemm_quad(const GemmArgs& a_in, int splits, hipStream_t st) {
   constexpr int COLS = (EPI == EPI_SILU) ? C::BF / 2 : C::BF;
   const int64_t worst = static_cast<int64_t>(a.num_t_blocks) * a.num_f_tiles;
   // After many whole rounds the workgroups are no longer in step (half tiles, hand-overs), and cutting the last
-  // round buys less than its slices' fp32 round trip costs: gate/up at 4096 / 16384 tokens (17 / 70 rounds) 1521 /
-  // 5743 us with the split, 1505 / 5723 without; the down projection (2.7 / 11 rounds) 785 against 915, 2803 / 2979.
-  const bool tail = a.tail_ws && a.K / BK >= kTailMinTiles && a.N % COLS == 0 && worst < 16 * static_cast<int64_t>(resident);
+  // round buys less than its slices' fp32 round trip costs - the sooner the shorter a tile's K loop is: gate/up
+  // (64 K tiles) with / without the split 681 / 684 us at 8.8 rounds (1536 tokens), 832 / 816 at 10.5, 1030 / 988
+  // at 12.5, 1521 / 1505 at 17.5, 5743 / 5723 at 70; the down projection (224 K tiles) 785 / 915 at 2.7 rounds,
+  // 2803 / 2979 at 11.
+  const int64_t max_rounds = a.K / BK >= 128 ? 16 : 8;
+  const bool tail = a.tail_ws && a.K / BK >= kTailMinTiles && a.N % COLS == 0 && worst < max_rounds * static_cast<int64_t>(resident);
   if (!tail) a.tail_ws = nullptr;
   int64_t grid = resident;
   if (tail) {
