@@ -95,6 +95,39 @@ def test_plan_table():
     assert p.tail_bytes == 0
 
 
+def test_plan_invariants_on_random_shapes():
+    """Whatever the shape, a plan is one the entry points can run: a routing block the kernels have, sorted_len as
+    moe_align_block_size lays it out (`ops/fused_moe.py:133-175` of the reference: n + E * (block - 1) slots), at least
+    one K slice and never more than the down projection has 128-byte K tiles, a workspace that holds the activated
+    rows and the routing arrays, the same answer whatever the weight layout flags, and shape errors as codes."""
+    import random
+    from fast_route_amd import _native
+    lib = _native.lib()
+    rng = random.Random(20240229)
+    p, q = _native.FrMoePlan(), _native.FrMoePlan()
+    for case in range(600):
+        dt = rng.choice([_native.FR_BF16, _native.FR_F16, _native.FR_FP8_E4M3])
+        mult = 256 if dt == _native.FR_FP8_E4M3 else 128
+        H, F = mult * rng.randint(1, 64), mult * rng.randint(1, 128)
+        E = rng.choice([1, 2, 3, 8, 16, 60, 64, 128, 256, 1022, 1024])
+        k = rng.randint(1, min(E, 8))
+        M = rng.choice([0, 1, 2, 4, 5, 16, 100, 1000, 5000, 40000, 300000, rng.randint(1, 1 << 20)])
+        where = "case %d: M=%d H=%d F=%d E=%d k=%d dtype=%d" % (case, M, H, F, E, k, dt)
+        assert lib.fr_moe_get_plan(M, H, F, E, k, dt, p) == 0, where
+        n, es = M * k, 1 if dt == _native.FR_FP8_E4M3 else 2
+        assert p.block in (16, 32, 64, 128, 160, 256), where
+        assert p.sorted_len == n + E * (p.block - 1), where
+        assert 1 <= p.split_k <= max(1, F * es // 128), where
+        assert 0 <= p.tail_bytes <= p.workspace_bytes, where
+        assert p.workspace_bytes >= p.sorted_len * F * es + 4 * (p.sorted_len + n + E), where
+        assert lib.fr_moe_get_plan(M, H, F, E, k, dt | _native.FR_W_TILED, q) == 0, where
+        assert (q.block, q.split_k, q.workspace_bytes) == (p.block, p.split_k, p.workspace_bytes), where
+        assert lib.fr_moe_get_plan(M, H + 64, F, E, k, dt, q) == -2, where
+        assert lib.fr_moe_get_plan(M, H, F, E, E + 1, dt, q) == -2, where
+    assert lib.fr_moe_get_plan(1 << 30, 4096, 14336, 8, 2, _native.FR_BF16, p) == -2
+    assert lib.fr_moe_get_plan(16, 4096, 14336, 1025, 2, _native.FR_BF16, p) == -2
+
+
 def test_ops_refuse_cpu_tensors():
     import torch
     from fast_route_amd.ops.fused_moe import moe_align_block_size
