@@ -53,6 +53,12 @@ constexpr int kQuadMinTiles = 8;    // K tiles per work unit, at least (two peel
 constexpr int kQuadTouchAhead = FQ_AHEAD;  // K tiles between a touch and the tile loads of the same rows
 constexpr int kQuadSink = 1024;     // bytes of LDS the touches land in (256 per wavefront)
 
+#ifndef FQ_TAIL_LONG_K  // measurement switches of the host side: K tiles from which a K loop counts as long, and
+#define FQ_TAIL_LONG_K 112
+#endif
+#ifndef FQ_TAIL_ROUNDS_SHORT  // whole rounds after which a shorter one stops splitting its last round
+#define FQ_TAIL_ROUNDS_SHORT 8
+#endif
 #ifndef FQ_XSHARE
 #define FQ_XSHARE 4
 #endif
@@ -520,8 +526,9 @@ int launch_gemm_quad(const GemmArgs& a_in, int splits, hipStream_t st) {
   // round buys less than its slices' fp32 round trip costs - the sooner the shorter a tile's K loop is: gate/up
   // (64 K tiles) with / without the split 681 / 684 us at 8.8 rounds (1536 tokens), 832 / 816 at 10.5, 1030 / 988
   // at 12.5, 1521 / 1505 at 17.5, 5743 / 5723 at 70; the down projection (224 K tiles) 785 / 915 at 2.7 rounds,
-  // 2803 / 2979 at 11.
-  const int64_t max_rounds = a.K / BK >= 128 ? 16 : 8;
+  // 2803 / 2979 at 11; fp8 down projection (112 K tiles) 1743 / 1794 at 8.5 rounds; 96 K tiles (H = 6144) 1138 / 1135
+  // at 10 rounds, 1442 / 1437 at 12.
+  const int64_t max_rounds = a.K / BK >= FQ_TAIL_LONG_K ? 16 : FQ_TAIL_ROUNDS_SHORT;
   const bool tail = a.tail_ws && a.K / BK >= kTailMinTiles && a.N % COLS == 0 && worst < max_rounds * static_cast<int64_t>(resident);
   if (!tail) a.tail_ws = nullptr;
   int64_t grid = resident;
